@@ -1,0 +1,200 @@
+"""Benchmark of the retention hot path on one MI355X.
+
+A step is one forward + backward of fused_chunk_retention over one synthetic batch of
+BASELINE config 2 (bf16, B=8 H=16 T=4096 dk=dv=128, zero initial state, dO ~ N(0,1)), inputs
+resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic FLOP count
+(dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the pass kernel measured
+with events on the launch stream, and the CPU oracle timed on the host cores beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "flash-pop_amd"), os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+CHUNK = 64
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def algorithmic_flops(B, T, H, dk, dv, C=CHUNK):
+    fwd = 2 * (C * (dk + dv) + 2 * dk * dv)
+    bwd = 2 * (C * (3 * dk + 2 * dv) + 4 * dk * dv)
+    n = B * T * H
+    return fwd * n, bwd * n
+
+
+def algorithmic_bytes(B, T, H, dk, dv):
+    n = B * T * H
+    return 2 * (2 * dk + 2 * dv) * n, 2 * (4 * dk + 3 * dv) * n
+
+
+def gpu_leg(args):
+    import torch
+    import oracle
+    import helpers as hp
+    from flash_pop_amd import fused_chunk_retention, flash_pop_retention, _lib
+
+    _lib.load()   # fail loudly before any timing if the HIP library is missing
+    dev = "cuda:0"
+    B, T, H, dk, dv = 8, 4096, 16, 128, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0, device=dev)
+    d_o, = hp.make_cotangents([(B, T, H, dv)], seed=1, device=dev)
+    leaves = [t.requires_grad_() for t in (q, k, v)]   # the state is the caller's zeros: no gradient
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        o, S = fused_chunk_retention(*leaves, s, decays)
+        if ev:
+            ev[1].record()
+        grads = torch.autograd.grad([o], leaves, [d_o])
+        if ev:
+            ev[2].record()
+        return grads
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    ms_per_step = wall * 1e3 / args.steps
+
+    f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
+    b_fwd, b_bwd = algorithmic_bytes(B, T, H, dk, dv)
+    tflops = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
+    # one step = 4 launches of the same pass kernel (fwd, dq, dk, dv)
+    launches = 4
+    avg_launch_ms = (fwd_ms + bwd_ms) / launches
+    achieved_gbs = (b_fwd + b_bwd) / launches / (avg_launch_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "fwd+bwd retention TFLOP/s, B=8 H=16 T=4096 d=128 bf16",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "config 2: chunked retention fwd+bwd, B=8 H=16 T=4096 dk=dv=128 chunk 64, bf16 in / fp32 accumulate"},
+        "tokens_per_s": round(B * T / (ms_per_step * 1e-3), 1),
+        "fwd_ms": round(fwd_ms, 4),
+        "bwd_ms": round(bwd_ms, 4),
+        "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "retention_pass_kernel<128>",
+            "achieved": round(achieved_gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "launches_per_step": launches,
+            "avg_launch_ms": round(avg_launch_ms, 4),
+            "algorithmic_bytes_per_launch": (b_fwd + b_bwd) // launches,
+        },
+    }
+
+    if not args.no_pop:
+        # POP (config 4): context through flash_pop_retention with 64-token blocks, 65 suffixes of
+        # 16 tokens per sequence through fused_chunk_retention from the block states.
+        block, Ls = 64, 16
+        N = T // block
+        qs, ks, vs, _ = hp.make_inputs(B * (N + 1), Ls, H, dk, dv, seed=2, device=dev)
+        d_os, = hp.make_cotangents([(B * (N + 1), Ls, H, dv)], seed=3, device=dev)
+        sleaves = [t.requires_grad_() for t in (qs, ks, vs)]
+
+        def pop_step():
+            o, states = flash_pop_retention(*leaves, s, decays, block)
+            starts = torch.cat((s[:, None], states), dim=1).flatten(0, 1)
+            o_s, _ = fused_chunk_retention(*sleaves, starts, decays)
+            return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
+
+        for _ in range(max(2, args.warmup // 4)):
+            pop_step()
+        torch.cuda.synchronize()
+        n = max(3, args.steps // 4)
+        t0 = time.perf_counter()
+        for _ in range(n):
+            pop_step()
+        torch.cuda.synchronize()
+        pop_ms = (time.perf_counter() - t0) * 1e3 / n
+        tok_ctx, tok_sfx = B * T, B * (N + 1) * Ls
+        out["pop"] = {
+            "workload": "config 4: POP context (64-token blocks) + 65 suffixes x 16 tokens per sequence, fwd+bwd",
+            "ms_per_step": round(pop_ms, 4),
+            "tokens": tok_ctx + tok_sfx,
+            "cost_per_token_vs_plain": round((pop_ms / (tok_ctx + tok_sfx)) / (ms_per_step / tok_ctx), 3),
+        }
+    return out
+
+
+def cpu_leg(sample_batch=1, reps=2):
+    """The oracle (chunk 64, fp32, torch autograd for the backward) on the host cores, on
+    `sample_batch` of the 8 sequences of config 2."""
+    import torch
+    import oracle
+    import helpers as hp
+
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    B, T, H, dk, dv = sample_batch, 4096, 16, 128, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0)
+    d_o, = hp.make_cotangents([(B, T, H, dv)], seed=1)
+    times = []
+    for i in range(reps + 1):
+        t0 = time.perf_counter()
+        hp.oracle_plain(q, k, v, s, decays, d_o, None, chunk=CHUNK)
+        if i:
+            times.append(time.perf_counter() - t0)
+    sec = sorted(times)[len(times) // 2]
+    f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
+    return {
+        "value": round((f_fwd + f_bwd) / sec / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{B} of the 8 sequences of config 2 (H=16 T=4096 d=128), fp32, chunk 64, fwd+bwd, "
+                  f"median of {reps} after 1 warm-up, {sec:.2f} s each",
+        "tokens_per_s": round(B * T / sec, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+    out = gpu_leg(args)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_leg()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

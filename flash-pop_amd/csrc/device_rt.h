@@ -1,0 +1,38 @@
+// Device primitives the pass kernel is written against (gfx950 / CDNA4).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define FP_DEVICE __device__ __forceinline__
+
+namespace fprt {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+FP_DEVICE int thread_index() { return threadIdx.x; }
+FP_DEVICE int block_index() { return blockIdx.x; }
+FP_DEVICE int grid_size() { return gridDim.x; }
+FP_DEVICE void block_sync() { __syncthreads(); }
+
+// D = A(32x16) * B(16x32) + C, bf16 inputs, fp32 accumulate (v_mfma_f32_32x32x16_bf16).
+// Lane l supplies A[l%32][8*(l/32) + e] and B[8*(l/32) + e][l%32], e = 0..7, and holds
+// D[8*(r/4) + 4*(l/32) + r%4][l%32] in element r.
+FP_DEVICE f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
+                                                 0, 0);
+}
+
+// Two floats -> two bf16 (round to nearest even), `lo` in bits 0..15 (v_cvt_pk_bf16_f32).
+FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
+FP_DEVICE float exp2_approx(float x) { return exp2f(x); }
+
+}  // namespace fprt

@@ -1,0 +1,58 @@
+// Arguments of one "retention pass" launch, shared by host and device code.
+//
+// Every kernel launch of this library is one instance of the same recurrence over the
+// tokens of each (batch, head) stream, in chunks of CH tokens of length L <= CH:
+//
+//   Y_i  = s_intra * sum_j m(i,j) (x_i . w_j) z_j  +  wread(i) * x_i R
+//   R   <- gamma^L R + sum_j wkey(j) w_j^T z_j
+//
+// forward in time (reverse == 0):  m = gamma^(i-j) [i >= j],  wread(i) = s_read   * gamma^(i+1),
+//                                  wkey(j) = s_update * gamma^(L-1-j)
+// backward in time (reverse == 1): m = gamma^(j-i) [j >= i],  wread(i) = s_read   * gamma^(L-1-i),
+//                                  wkey(j) = s_update * gamma^(j+1)
+//
+// X, W are [B, T, H, dA]; Z, Y are [B, T, H, dB]; R is a dA x dB matrix per (b, h) kept in
+// fp32 registers for the whole sequence.  The retention forward and its three gradient
+// passes are four choices of (X, W, Z, R); see flashpop_api.cpp.
+#pragma once
+#include <stdint.h>
+
+namespace fpk {
+
+constexpr int CH = 64;          // tokens per chunk
+constexpr int BV = 64;          // columns of Z / Y / R owned by one workgroup
+constexpr int NTHREADS = 256;   // 4 wave64
+constexpr int MAX_HEADS = 128;
+
+struct PassArgs {
+  const uint16_t* X;
+  const uint16_t* W;
+  const uint16_t* Z;
+  uint16_t* Y;
+  const uint16_t* R0;    // initial R per (b, h), nullable (zeros)
+  uint16_t* Rout;        // final R per (b, h), nullable
+  uint16_t* Bout;        // R after every full block, [B, nblk, H, dk*dv], nullable (forward only)
+  const uint16_t* Bin;   // added to R before the chunk that ends each full block, nullable (reverse only)
+  long long rs_a, rs_n;  // element strides of R[a][n] inside one dk*dv state matrix
+  int B, T, H, dA, dB;
+  int nblk;              // number of full blocks (T / block), 0 if block == 0
+  int block;             // block size in tokens; chunks never straddle a multiple of it (0: none)
+  int reverse;
+  float s_intra, s_read, s_update;
+  float log2g[MAX_HEADS];
+};
+
+// LDS bytes the pass kernel needs for a given dA.
+constexpr int lds_bytes(int dA) {
+  return 2 * (2 * CH * (dA + 8)      // X and W tiles, row-major
+              + dA * (CH + 4)        // weighted W, transposed
+              + BV * (CH + 4)        // Z, transposed
+              + BV * (dA + 8)        // bf16 copy of R, transposed
+              + CH * (BV + 8));      // Y staging
+}
+
+}  // namespace fpk
+
+// Launches the pass kernel on `stream` (a hipStream_t, or ignored by the CPU test harness).
+// Returns 0 on success; on failure returns nonzero and *err points at a static message.
+int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err);

@@ -1,0 +1,57 @@
+"""ctypes binding of libflashpop_hip.so (declarations: include/flashpop_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_void_p, POINTER, c_double
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libflashpop_hip.so"
+LIB_PATH = os.path.join(_HERE, LIB_NAME)
+
+_P, _I = c_void_p, c_int
+_D = POINTER(c_double)
+
+# name -> argument types, in the order of include/flashpop_hip.h
+SIGNATURES = {
+    "fp_retention_fwd": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P],
+    "fp_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "fp_pop_retention_fwd": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "fp_pop_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "fp_last_error": [],
+    "fp_version": [],
+}
+
+_lib = None
+
+
+def bind(path: str) -> ctypes.CDLL:
+    """Open a library exporting the flashpop C ABI and declare its prototypes."""
+    lib = ctypes.CDLL(path)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is missing
+        fn.argtypes = argtypes
+        fn.restype = c_char_p if name == "fp_last_error" else c_int
+    return lib
+
+
+def load() -> ctypes.CDLL:
+    """The HIP library built in-tree.  There is no fallback: a missing library is an error."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it first (python flash-pop_amd/build.py, or "
+                "__graft_entry__.build()). flash_pop_amd has no non-HIP execution path.")
+        _lib = bind(LIB_PATH)
+    return _lib
+
+
+def decays_array(head_decays) -> ctypes.Array:
+    vals = [float(g) for g in head_decays]
+    return (c_double * len(vals))(*vals)
+
+
+def check(lib: ctypes.CDLL, rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(f"flashpop_hip error {rc}: {lib.fp_last_error().decode()}")

@@ -1,0 +1,81 @@
+"""Tensor-level plumbing shared by the two autograd Functions: checks, allocation, raw calls."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def prepare(q, k, v, s, head_decays):
+    """Validate like the reference's asserts (fused_retention/__init__.py:20,
+    pop_retention/__init__.py:17-18) and return contiguous tensors plus the shape."""
+    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
+        raise ValueError(f"expected q, k [B,T,H,dk] and v [B,T,H,dv]; got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    assert len(head_decays) == H, f"got {len(head_decays)} head decays for {H} heads"
+    for name, t in (("q", q), ("k", k), ("v", v), ("s", s)):
+        if t is None:
+            continue
+        assert t.dtype == torch.bfloat16, f"{name}: only bfloat16 is supported, got {t.dtype}"
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}: flash_pop_amd runs on the GPU only")
+    if s is not None and tuple(s.shape) != (B, H, dk, dv):
+        raise ValueError(f"expected state [B,H,dk,dv] = {(B, H, dk, dv)}, got {tuple(s.shape)}")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    s = None if s is None else s.contiguous()
+    return q, k, v, s, (B, T, H, dk, dv)
+
+
+def retention_fwd(q, k, v, s, decays, shape):
+    lib = _lib.load()
+    B, T, H, dk, dv = shape
+    o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
+    s_out = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.fp_retention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o), _ptr(s_out),
+                                  B, T, H, dk, dv, _stream())
+    _lib.check(lib, rc)
+    return o, s_out
+
+
+def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
+    lib = _lib.load()
+    B, T, H, dk, dv = shape
+    o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
+    states = torch.empty((B, T // block_size, H, dk, dv), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.fp_pop_retention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
+                                      _ptr(states) if states.numel() else None, B, T, H, dk, dv, block_size, _stream())
+    _lib.check(lib, rc)
+    return o, states
+
+
+def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0):
+    """Gradients for both ops; block_size is None for the plain op."""
+    lib = _lib.load()
+    B, T, H, dk, dv = shape
+    d_o = d_o.contiguous()
+    d_s_out = None if d_s_out is None else d_s_out.contiguous()
+    d_blocks = None if d_blocks is None or d_blocks.numel() == 0 else d_blocks.contiguous()
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    d_s0 = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device) if want_ds0 else None
+    with torch.cuda.device(q.device):
+        if block_size is None:
+            rc = lib.fp_retention_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
+                                      _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
+                                      _stream())
+        else:
+            rc = lib.fp_pop_retention_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
+                                          _ptr(d_blocks), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
+                                          block_size, _stream())
+    _lib.check(lib, rc)
+    return dq, dk_, dv_, d_s0

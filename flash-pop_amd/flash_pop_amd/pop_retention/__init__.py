@@ -1,0 +1,37 @@
+"""flash_pop_retention(q, k, v, s, head_decays, block_size) -> (o, block_states)
+
+Same call signature and returns as the reference's FlashPOPRetention
+(flash_pop/pop_retention/__init__.py:11-52): block_states is [B, T // block_size, H, dk, dv],
+the recurrent state after every full block; there is no final-state output.  The block size
+is kept on the autograd context, so T need not be a multiple of it in the backward pass
+(the reference re-derives it as T // num_blocks, pop_retention/__init__.py:39-40).
+"""
+import torch
+
+from .. import _ops
+
+
+class FlashPOPRetention(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, q, k, v, s, head_decays, block_size):
+        block_size = int(block_size)
+        assert block_size >= 1, f"block_size must be positive, got {block_size}"
+        q, k, v, s, shape = _ops.prepare(q, k, v, s, head_decays)
+        o, states = _ops.pop_retention_fwd(q, k, v, s, head_decays, block_size, shape)
+        ctx.save_for_backward(q, k, v, s)
+        ctx.head_decays = tuple(head_decays)
+        ctx.shape = shape
+        ctx.block_size = block_size
+        return o, states
+
+    @staticmethod
+    def backward(ctx, d_o, d_block_states):
+        q, k, v, s = ctx.saved_tensors
+        want_ds0 = s is not None and ctx.needs_input_grad[3]
+        dq, dk, dv, d_s0 = _ops.retention_bwd(q, k, v, s, ctx.head_decays, ctx.shape, d_o, None, d_block_states,
+                                              ctx.block_size, want_ds0)
+        return dq, dk, dv, d_s0, None, None
+
+
+flash_pop_retention = FlashPOPRetention.apply

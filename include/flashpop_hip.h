@@ -1,0 +1,78 @@
+/* flashpop_hip.h -- C ABI of libflashpop_hip.so: fused chunked retention and POP retention
+ * on AMD MI355X (gfx950).
+ *
+ * The reference has no native ABI for this path: its "ABI" is a TileLang JIT kernel object
+ * called from two torch.autograd.Functions.  Each entry point below replaces the kernel
+ * launches inside one of those four methods; the citation names that method.
+ *
+ * Conventions common to all entry points
+ *   - every tensor pointer is DEVICE memory, bf16 (2 bytes/element), contiguous, in the
+ *     reference's layouts: q, k, dq, dk [B,T,H,dk]; v, o, d_o, dv [B,T,H,dv]; states
+ *     [B,H,dk,dv]; block states [B, T/block_size, H, dk, dv]
+ *   - head_decays is HOST memory: H doubles, gamma_h in (0, 1]
+ *   - K is divided by sqrt(dk) inside (flash_pop/fused_retention/reference.py:57); Q is not scaled
+ *   - dk, dv in {64, 128, 256}; 1 <= H <= 128; T >= 1; B >= 1
+ *   - the caller owns every buffer; the library allocates nothing and keeps no pointer
+ *   - launches are asynchronous on `stream` (a hipStream_t, NULL = default stream)
+ *   - returns 0 on success, a negative FP_ERR_* code otherwise; fp_last_error() then gives a
+ *     message (thread-local).  No kernel is launched when an argument check fails.
+ *   - results are deterministic: no atomics, fixed reduction order
+ */
+#ifndef FLASHPOP_HIP_H
+#define FLASHPOP_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP_OK 0
+#define FP_ERR_NULL_POINTER (-1)
+#define FP_ERR_BAD_SHAPE (-2)
+#define FP_ERR_UNSUPPORTED_DIM (-3)
+#define FP_ERR_BAD_DECAY (-4)
+#define FP_ERR_LAUNCH (-5)
+
+/* Replaces the kernel call in FusedChunkRetention.forward
+ * (flash_pop/fused_retention/__init__.py:13-31).
+ *   s0     initial state, may be NULL (zeros)
+ *   o      out: retention output
+ *   s_out  out: state after the last token, may be NULL */
+int fp_retention_fwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                     void* o, void* s_out, int B, int T, int H, int dk, int dv, void* stream);
+
+/* Replaces the two kernel calls and four reductions in FusedChunkRetention.backward
+ * (flash_pop/fused_retention/__init__.py:34-47).
+ *   d_o      gradient of o
+ *   d_s_out  gradient of the final state, may be NULL (zeros)
+ *   dq, dk_, dv_  out: gradients of q, k (unscaled), v
+ *   d_s0     out: gradient of the initial state, may be NULL (not wanted) */
+int fp_retention_bwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                     const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B, int T,
+                     int H, int dk, int dv, void* stream);
+
+/* Replaces the kernel call in FlashPOPRetention.forward
+ * (flash_pop/pop_retention/__init__.py:14-31).
+ *   block_states  out: state after every FULL block of block_size tokens,
+ *                 [B, T / block_size, H, dk, dv]; may be NULL only if T < block_size */
+int fp_pop_retention_fwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                         void* o, void* block_states, int B, int T, int H, int dk, int dv, int block_size,
+                         void* stream);
+
+/* Replaces the two kernel calls and four reductions in FlashPOPRetention.backward
+ * (flash_pop/pop_retention/__init__.py:34-50).  block_size is passed explicitly (the
+ * reference infers it as T / num_blocks, which is wrong when T % block_size != 0).
+ *   d_block_states  gradient of block_states, may be NULL (zeros) */
+int fp_pop_retention_bwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                         const void* d_o, const void* d_block_states, void* dq, void* dk_, void* dv_, void* d_s0,
+                         int B, int T, int H, int dk, int dv, int block_size, void* stream);
+
+/* Message for the last nonzero return on this thread ("" if none). */
+const char* fp_last_error(void);
+
+/* ABI version: major * 1000 + minor. */
+int fp_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHPOP_HIP_H */

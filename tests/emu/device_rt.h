@@ -1,0 +1,79 @@
+// CPU stand-in for the device primitives: one OS thread per GPU lane, pthread barriers for
+// workgroup and wave synchronisation, MFMA evaluated from the documented lane layout.
+// Test infrastructure only: lets the kernel body run under ASan / gdb and be compared with
+// the oracle without a GPU.  Never part of the shipped library.
+#pragma once
+#include <pthread.h>
+#include <stdint.h>
+
+#include <cmath>
+#include <cstring>
+
+#define FP_DEVICE inline __attribute__((always_inline))
+
+namespace fprt {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct WaveShared {
+  uint16_t A[64][8];
+  uint16_t Bm[64][8];
+  pthread_barrier_t bar;
+};
+
+struct LaneCtx {
+  int tid, block, grid;
+  WaveShared* wave;
+  pthread_barrier_t* wg_bar;
+};
+
+extern thread_local LaneCtx g_lane;
+
+FP_DEVICE int thread_index() { return g_lane.tid; }
+FP_DEVICE int block_index() { return g_lane.block; }
+FP_DEVICE int grid_size() { return g_lane.grid; }
+FP_DEVICE void block_sync() { pthread_barrier_wait(g_lane.wg_bar); }
+
+FP_DEVICE float bf16_to_f32(uint16_t b) {
+  uint32_t u = (uint32_t)b << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+FP_DEVICE uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);   // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+FP_DEVICE f32x16 mfma_32x32x16_bf16(u32x4 a, u32x4 b, f32x16 c) {
+  WaveShared* w = g_lane.wave;
+  const int lane = g_lane.tid & 63;
+  std::memcpy(w->A[lane], &a, 16);
+  std::memcpy(w->Bm[lane], &b, 16);
+  pthread_barrier_wait(&w->bar);
+  const int g = lane >> 5, n = lane & 31;
+  for (int r = 0; r < 16; ++r) {
+    const int m = 8 * (r >> 2) + 4 * g + (r & 3);
+    float acc = c[r];
+    for (int k = 0; k < 16; ++k) {
+      acc += bf16_to_f32(w->A[m + 32 * (k >> 3)][k & 7]) * bf16_to_f32(w->Bm[n + 32 * (k >> 3)][k & 7]);
+    }
+    c[r] = acc;
+  }
+  pthread_barrier_wait(&w->bar);
+  return c;
+}
+
+FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_rne(lo) | ((uint32_t)f32_to_bf16_rne(hi) << 16);
+}
+
+FP_DEVICE float exp2_approx(float x) { return std::exp2(x); }
+
+}  // namespace fprt

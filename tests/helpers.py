@@ -1,0 +1,154 @@
+"""Shared by the CPU-harness tests and the GPU parity tests: seeded inputs, oracle results
+on the bf16-rounded inputs, raw C-ABI calls, and the comparison bar."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+import oracle
+
+BF16 = torch.bfloat16
+
+# BASELINE tolerance for bf16 (rtol = atol = 2e-2) and the reference's own bar for outputs and
+# states, RMS(err)/RMS(ref) < 0.005 (tests/test_fused_retention.py:119,131).
+RTOL = 2e-2
+ATOL = 2e-2
+RMS_BAR = 5e-3
+
+
+def make_inputs(B, T, H, dk, dv, seed=0, state_std=None, device="cpu"):
+    """q, k, v ~ N(0,1) in bf16, generated on the CPU so every backend sees the same bits.
+    state_std: None -> no initial state; 0 -> zeros; else N(0, std^2)."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, T, H, dk, generator=g).to(BF16)
+    k = torch.randn(B, T, H, dk, generator=g).to(BF16)
+    v = torch.randn(B, T, H, dv, generator=g).to(BF16)
+    if state_std is None:
+        s = None
+    elif state_std == 0:
+        s = torch.zeros(B, H, dk, dv, dtype=BF16)
+    else:
+        s = (torch.randn(B, H, dk, dv, generator=g) * state_std).to(BF16)
+    mv = lambda t: None if t is None else t.to(device)
+    return mv(q), mv(k), mv(v), mv(s)
+
+
+def make_cotangents(shapes, seed=1, device="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(*s, generator=g).to(BF16).to(device) for s in shapes]
+
+
+def oracle_plain(q, k, v, s, decays, d_o=None, d_s=None, chunk=64, dtype=torch.float32):
+    """Oracle forward (and autograd backward) on the bf16-rounded inputs, computed in `dtype`."""
+    ins = [None if t is None else t.detach().cpu().to(dtype).requires_grad_(d_o is not None) for t in (q, k, v, s)]
+    o, S = oracle.chunkwise_retention(*ins, decays, chunk_size=chunk)
+    if d_o is None:
+        return o, S
+    loss = (o * d_o.cpu().to(dtype)).sum()
+    if d_s is not None:
+        loss = loss + (S * d_s.cpu().to(dtype)).sum()
+    grads = torch.autograd.grad(loss, [t for t in ins if t is not None])
+    if ins[3] is None:
+        grads = (*grads, None)
+    return o.detach(), S.detach(), grads
+
+
+def oracle_pop(q, k, v, s, decays, block, d_o=None, d_states=None, dtype=torch.float32):
+    ins = [None if t is None else t.detach().cpu().to(dtype).requires_grad_(d_o is not None) for t in (q, k, v, s)]
+    o, states = oracle.pop_retention(*ins, decays, block)
+    if d_o is None:
+        return o, states
+    loss = (o * d_o.cpu().to(dtype)).sum()
+    if d_states is not None and states.numel():
+        loss = loss + (states * d_states.cpu().to(dtype)).sum()
+    grads = torch.autograd.grad(loss, [t for t in ins if t is not None])
+    if ins[3] is None:
+        grads = (*grads, None)
+    return o.detach(), states.detach(), grads
+
+
+def error_report(got, ref):
+    got, ref = got.detach().cpu().double(), ref.detach().cpu().double()
+    err = (got - ref).abs()
+    rms_ref = ref.square().mean().sqrt().item()
+    return {
+        "rms_ratio": (err.square().mean().sqrt().item() / max(rms_ref, 1e-300)),
+        "max_abs": err.max().item() if err.numel() else 0.0,
+        "rms_ref": rms_ref,
+        "frac_outside": (err > ATOL + RTOL * ref.abs()).double().mean().item() if err.numel() else 0.0,
+    }
+
+
+def assert_close(got, ref, name, rms_bar=RMS_BAR):
+    """The parity bar.  Elementwise |got - ref| <= atol + rtol |ref| with rtol = 2e-2 and
+    atol = 2e-2 * max(1, RMS(ref)), plus RMS(err)/RMS(ref) < 0.005.  atol follows the tensor's
+    scale because the inputs are N(0,1) and not normalised: retention sums grow like the square
+    root of the retention window, and any bf16-operand evaluation (the reference's included)
+    carries an absolute error proportional to that scale, whatever the individual element's size."""
+    assert got.shape == ref.shape, f"{name}: shape {tuple(got.shape)} != {tuple(ref.shape)}"
+    if ref.numel() == 0:
+        return
+    rep = error_report(got, ref)
+    g, r = got.detach().cpu().double(), ref.detach().cpu().double()
+    assert torch.isfinite(g).all(), f"{name}: non-finite values"
+    atol = ATOL * max(1.0, rep["rms_ref"])
+    bad = (g - r).abs() > atol + RTOL * r.abs()
+    assert not bad.any(), f"{name}: {int(bad.sum())} of {bad.numel()} outside rtol={RTOL} atol={atol:.3g}; {rep}"
+    assert rep["rms_ratio"] < rms_bar, f"{name}: RMS error ratio {rep['rms_ratio']:.3g} >= {rms_bar}; {rep}"
+
+
+# ---- raw C-ABI calls (work on any device the library understands) --------------------------
+
+def _p(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _dec(decays):
+    return (ctypes.c_double * len(decays))(*[float(x) for x in decays])
+
+
+def _check(lib, rc):
+    assert rc == 0, f"rc={rc}: {lib.fp_last_error().decode()}"
+
+
+def raw_fwd(lib, q, k, v, s, decays, stream=None, want_state=True):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    o = torch.full((B, T, H, dv), float("nan"), dtype=BF16, device=q.device)
+    S = torch.full((B, H, dk, dv), float("nan"), dtype=BF16, device=q.device) if want_state else None
+    _check(lib, lib.fp_retention_fwd(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o), _p(S), B, T, H, dk, dv, stream))
+    return o, S
+
+
+def raw_bwd(lib, q, k, v, s, decays, d_o, d_s, stream=None, want_ds0=True):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    nan = lambda *shape: torch.full(shape, float("nan"), dtype=BF16, device=q.device)
+    dq, dk_, dv_ = nan(*q.shape), nan(*k.shape), nan(*v.shape)
+    ds0 = nan(B, H, dk, dv) if want_ds0 else None
+    _check(lib, lib.fp_retention_bwd(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(d_o), _p(d_s), _p(dq), _p(dk_),
+                                     _p(dv_), _p(ds0), B, T, H, dk, dv, stream))
+    return dq, dk_, dv_, ds0
+
+
+def raw_pop_fwd(lib, q, k, v, s, decays, block, stream=None):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    o = torch.full((B, T, H, dv), float("nan"), dtype=BF16, device=q.device)
+    states = torch.full((B, T // block, H, dk, dv), float("nan"), dtype=BF16, device=q.device)
+    _check(lib, lib.fp_pop_retention_fwd(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o),
+                                         _p(states) if states.numel() else None, B, T, H, dk, dv, block, stream))
+    return o, states
+
+
+def raw_pop_bwd(lib, q, k, v, s, decays, block, d_o, d_states, stream=None, want_ds0=True):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    nan = lambda *shape: torch.full(shape, float("nan"), dtype=BF16, device=q.device)
+    dq, dk_, dv_ = nan(*q.shape), nan(*k.shape), nan(*v.shape)
+    ds0 = nan(B, H, dk, dv) if want_ds0 else None
+    dst = d_states if d_states is not None and d_states.numel() else None
+    _check(lib, lib.fp_pop_retention_bwd(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(d_o), _p(dst), _p(dq), _p(dk_),
+                                         _p(dv_), _p(ds0), B, T, H, dk, dv, block, stream))
+    return dq, dk_, dv_, ds0

@@ -1,0 +1,72 @@
+"""The C-ABI library loads, exports every symbol include/flashpop_hip.h declares, and rejects
+bad arguments before touching a GPU (so these run on a CPU-only machine)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flashpop_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from flash_pop_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    return _lib.load()
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree(lib):
+    from flash_pop_amd import _lib
+    names = declared_functions()
+    assert names == sorted(_lib.SIGNATURES), (names, sorted(_lib.SIGNATURES))
+    for n in names:
+        assert hasattr(lib, n), f"{n} not exported"
+    assert lib.fp_version() == 1000
+
+
+def test_argument_checks_return_codes(lib):
+    dec = (ctypes.c_double * 2)(0.9, 0.95)
+    p = ctypes.c_void_p(0x1000)   # never dereferenced: every call below fails its checks first
+    null = None
+    ok_dims = (1, 8, 2, 64, 64)
+    assert lib.fp_retention_fwd(null, p, p, null, dec, p, null, *ok_dims, None) == -1
+    assert b"NULL" in lib.fp_last_error()
+    assert lib.fp_retention_fwd(p, p, p, null, None, p, null, *ok_dims, None) == -1
+    assert lib.fp_retention_fwd(p, p, p, null, dec, p, null, 1, 0, 2, 64, 64, None) == -2
+    assert lib.fp_retention_fwd(p, p, p, null, dec, p, null, 1, 8, 2, 96, 64, None) == -3
+    assert b"dk and dv" in lib.fp_last_error()
+    assert lib.fp_retention_fwd(p, p, p, null, dec, p, null, 1, 8, 2, 64, 32, None) == -3
+    bad = (ctypes.c_double * 2)(0.9, 1.5)
+    assert lib.fp_retention_fwd(p, p, p, null, bad, p, null, *ok_dims, None) == -4
+    bad0 = (ctypes.c_double * 2)(0.0, 0.5)
+    assert lib.fp_retention_fwd(p, p, p, null, bad0, p, null, *ok_dims, None) == -4
+    assert lib.fp_retention_bwd(p, p, p, null, dec, null, null, p, p, p, null, *ok_dims, None) == -1
+    assert lib.fp_pop_retention_fwd(p, p, p, null, dec, p, p, *ok_dims, 0, None) == -2
+    assert lib.fp_pop_retention_fwd(p, p, p, null, dec, p, null, *ok_dims, 4, None) == -1
+    assert lib.fp_pop_retention_bwd(p, p, p, null, dec, p, p, p, p, null, null, *ok_dims, 4, None) == -1
+    big = (ctypes.c_double * 200)(*([0.9] * 200))
+    assert lib.fp_retention_fwd(p, p, p, null, big, p, null, 1, 8, 200, 64, 64, None) == -2
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+    from flash_pop_amd import fused_chunk_retention, flash_pop_retention
+    q = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        fused_chunk_retention(q, q, q, None, (0.9, 0.9))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        flash_pop_retention(q, q, q, None, (0.9, 0.9), 4)
+    with pytest.raises(AssertionError, match="bfloat16"):
+        fused_chunk_retention(q.float(), q.float(), q.float(), None, (0.9, 0.9))
+    with pytest.raises(AssertionError, match="head decays"):
+        fused_chunk_retention(q, q, q, None, (0.9,))

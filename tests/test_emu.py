@@ -1,0 +1,87 @@
+"""Runs the real kernel body and the real C-ABI layer on the CPU (one OS thread per GPU lane,
+tests/emu/) and compares with the oracle.  This checks indexing, chunk scheduling, the pass
+mapping and ragged/unaligned handling without a GPU; it assumes the documented MFMA lane
+layout, which only the GPU parity tests can confirm."""
+import os
+import subprocess
+
+import pytest
+import torch
+
+import helpers as hp
+import oracle
+
+EMU_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu")
+
+
+@pytest.fixture(scope="module")
+def emu_lib():
+    subprocess.run([os.path.join(EMU_DIR, "build_emu.sh")], check=True)
+    from flash_pop_amd import _lib
+    return _lib.bind(os.path.join(EMU_DIR, "libflashpop_emu.so"))
+
+
+def _check_all(pairs):
+    for name, got, ref in pairs:
+        if ref is not None:
+            hp.assert_close(got, ref, name)
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,state_std", [
+    (1, 150, 2, 128, 128, 0.5),     # ragged tail, initial state
+    (1, 100, 2, 64, 128, None),     # dk != dv, no initial state
+    (2, 64, 1, 128, 64, 0.0),       # exactly one chunk, zero state
+    (1, 70, 1, 256, 64, 0.3),       # widest contraction
+    (1, 5, 3, 64, 64, 0.5),         # shorter than a chunk
+])
+def test_plain_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std):
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T, state_std=state_std)
+    d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=T + 1)
+    o, S = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+    dq, dk_, dv_, ds0 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
+    o_ref, S_ref, (gq, gk, gv, gs) = hp.oracle_plain(q, k, v, s, decays, d_o, d_s)
+    _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,block", [
+    (1, 150, 2, 128, 128, 64),      # block == chunk
+    (1, 287, 1, 64, 128, 144),      # block > chunk, ragged last block (reference generation shape)
+    (2, 28, 1, 64, 64, 15),         # block < chunk
+    (1, 130, 1, 64, 64, 32),        # block divides chunk
+    (1, 40, 1, 64, 64, 100),        # no full block at all
+])
+def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
+    decays = oracle.head_decays(H, (5, 12))
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + block, state_std=0.5)
+    d_o, d_b = hp.make_cotangents([(B, T, H, dv), (B, T // block, H, dk, dv)], seed=T)
+    o, states = hp.raw_pop_fwd(emu_lib, q, k, v, s, decays, block)
+    dq, dk_, dv_, ds0 = hp.raw_pop_bwd(emu_lib, q, k, v, s, decays, block, d_o, d_b)
+    o_ref, st_ref, (gq, gk, gv, gs) = hp.oracle_pop(q, k, v, s, decays, block, d_o, d_b)
+    _check_all([("o", o, o_ref), ("states", states, st_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv),
+                ("ds0", ds0, gs)])
+
+
+def test_optional_outputs_and_determinism(emu_lib):
+    decays = oracle.head_decays(2)
+    q, k, v, s = hp.make_inputs(1, 90, 2, 64, 64, seed=3, state_std=0.5)
+    o1, S1 = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+    o2, none = hp.raw_fwd(emu_lib, q, k, v, s, decays, want_state=False)
+    assert none is None and torch.equal(o1, o2)
+    d_o, = hp.make_cotangents([(1, 90, 2, 64)], seed=4)
+    g1 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None)
+    g2 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None, want_ds0=False)
+    assert g2[3] is None and all(torch.equal(a, b) for a, b in zip(g1[:3], g2[:3]))
+    z = torch.zeros(1, 2, 64, 64, dtype=hp.BF16)
+    g3 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, z)
+    assert all(torch.equal(a, b) for a, b in zip(g1, g3))
+
+
+def test_gamma_one_and_tiny(emu_lib):
+    """gamma = 1 (no decay) and a gamma small enough that gamma^63 underflows."""
+    decays = (1.0, 1e-3)
+    q, k, v, s = hp.make_inputs(1, 130, 2, 64, 64, seed=9, state_std=0.5)
+    o, S = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+    o_ref, S_ref = hp.oracle_plain(q, k, v, s, decays)
+    hp.assert_close(o, o_ref, "o")
+    hp.assert_close(S, S_ref, "S")

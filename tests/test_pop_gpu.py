@@ -1,0 +1,113 @@
+"""GPU parity tests for flash_pop_retention and the POP suffix path, through the C ABI.
+Same bar as test_retention_gpu.py."""
+import pytest
+import torch
+
+import helpers as hp
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def run_pop(B, T, H, dk, dv, block, state_std, seed, decay_range=(5, 12), oracle_batches=None):
+    from flash_pop_amd import flash_pop_retention
+    _say(f"[pop] B{B} T{T} H{H} dk{dk} dv{dv} block={block} s0={state_std} seed={seed}")
+    decays = oracle.head_decays(H, decay_range)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=seed, state_std=state_std)
+    d_o, d_b = hp.make_cotangents([(B, T, H, dv), (B, T // block, H, dk, dv)], seed=seed + 1)
+    leaves = [None if t is None else t.to(DEV).requires_grad_() for t in (q, k, v, s)]
+    o, states = flash_pop_retention(*leaves, decays, block)
+    assert states.shape == (B, T // block, H, dk, dv) and states.dtype == torch.bfloat16
+    torch.autograd.backward([o, states], [d_o.to(DEV), d_b.to(DEV)])
+    torch.cuda.synchronize()
+    for b in (range(B) if oracle_batches is None else oracle_batches):
+        sl = slice(b, b + 1)
+        o_ref, st_ref, grads = hp.oracle_pop(q[sl], k[sl], v[sl], None if s is None else s[sl], decays, block,
+                                             d_o[sl], d_b[sl])
+        hp.assert_close(o[sl], o_ref, f"o[b={b}]")
+        hp.assert_close(states[sl], st_ref, f"states[b={b}]")
+        for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), leaves, grads):
+            if ref is not None:
+                hp.assert_close(leaf.grad[sl], ref, f"{name}[b={b}]")
+    return o, states
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,block", [
+    (4, 287, 4, 64, 128, 144),     # generation scenario (tests/test_pop_retention.py:161-181)
+    (4, 28, 4, 64, 128, 15),       # block shorter than a chunk (:183-196)
+    (2, 640, 4, 64, 128, 32),      # training scenario (:216-230)
+    (2, 300, 4, 64, 128, 15),      # (:232-246)
+    (2, 512, 4, 64, 64, 500),      # reference bwd test shape (:249-262): T % block != 0
+    (2, 1440, 4, 64, 128, 144),    # 10 blocks of 144
+    (2, 256, 2, 128, 128, 64),     # block == chunk, headline head dims
+    (1, 40, 2, 64, 64, 100),       # no full block: empty block_states
+    (1, 192, 2, 128, 256, 64),
+])
+def test_pop_parity_sweep(B, T, H, dk, dv, block):
+    run_pop(B, T, H, dk, dv, block, 0.3, seed=T + block)
+
+
+def test_pop_without_state_argument():
+    run_pop(2, 130, 2, 64, 64, 64, None, seed=4)
+
+
+def test_pop_outputs_equal_plain_outputs():
+    """The context outputs of the POP op are those of the plain op (same chunk partition when
+    block is a chunk multiple -> bit-identical), and its last block state is the plain final state."""
+    from flash_pop_amd import flash_pop_retention, fused_chunk_retention
+    B, T, H, d, block = 2, 1024, 4, 128, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=21, state_std=0.1, device=DEV)
+    o_pop, states = flash_pop_retention(q, k, v, s, decays, block)
+    o, S = fused_chunk_retention(q, k, v, s, decays)
+    assert torch.equal(o_pop, o) and torch.equal(states[:, -1], S)
+
+
+def _suffix_case(B, N, block, Ls, H, dk, dv, seed, oracle_batches):
+    """Context through flash_pop_retention, N + 1 suffixes per sequence through
+    fused_chunk_retention started from [S0, block states] (flash_pop/pop_retnet.py:152-171),
+    gradients chained through both ops by autograd."""
+    from flash_pop_amd import flash_pop_retention, fused_chunk_retention
+    T = N * block
+    _say(f"[pop+suffix] B{B} N{N} block{block} Ls{Ls} H{H} dk{dk} dv{dv}")
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=seed, state_std=0.05)
+    qs, ks, vs, _ = hp.make_inputs(B * (N + 1), Ls, H, dk, dv, seed=seed + 1)
+    d_o, d_os = hp.make_cotangents([(B, T, H, dv), (B * (N + 1), Ls, H, dv)], seed=seed + 2)
+    ctx_leaves = [t.to(DEV).requires_grad_() for t in (q, k, v, s)]
+    sfx_leaves = [t.to(DEV).requires_grad_() for t in (qs, ks, vs)]
+    o, states = flash_pop_retention(*ctx_leaves, decays, block)
+    starts = torch.cat((ctx_leaves[3][:, None], states), dim=1).flatten(0, 1)
+    o_sfx, _ = fused_chunk_retention(*sfx_leaves, starts, decays)
+    torch.autograd.backward([o, o_sfx], [d_o.to(DEV), d_os.to(DEV)])
+    torch.cuda.synchronize()
+
+    for b in oracle_batches:
+        sl, ssl = slice(b, b + 1), slice(b * (N + 1), (b + 1) * (N + 1))
+        ins = [t[sl].float().requires_grad_() for t in (q, k, v, s)]
+        sins = [t[ssl].float().requires_grad_() for t in (qs, ks, vs)]
+        o_ref, st_ref = oracle.pop_retention(*ins, decays, block)
+        os_ref = oracle.pop_suffix_retention(*sins, ins[3], st_ref, decays)
+        loss = (o_ref * d_o[sl].float()).sum() + (os_ref * d_os[ssl].float()).sum()
+        grads = torch.autograd.grad(loss, ins + sins)
+        hp.assert_close(o[sl], o_ref.detach(), "ctx o")
+        hp.assert_close(o_sfx[ssl], os_ref.detach(), "suffix o")
+        for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), ctx_leaves, grads[:4]):
+            hp.assert_close(leaf.grad[sl], ref, f"ctx {name}")
+        for name, leaf, ref in zip(("dq", "dk", "dv"), sfx_leaves, grads[4:]):
+            hp.assert_close(leaf.grad[ssl], ref, f"suffix {name}")
+
+
+def test_pop_suffix_path_small():
+    _suffix_case(B=2, N=3, block=32, Ls=8, H=2, dk=64, dv=64, seed=30, oracle_batches=[0, 1])
+
+
+def test_config4_pop_with_suffixes():
+    """BASELINE config 4: B8 H16 d128, T4096 in 64-token blocks, 16-token suffixes at every boundary
+    (N + 1 = 65 per sequence, the first from S0).  Oracle on one sequence."""
+    _suffix_case(B=8, N=64, block=64, Ls=16, H=16, dk=128, dv=128, seed=40, oracle_batches=[5])

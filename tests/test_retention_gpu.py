@@ -1,0 +1,163 @@
+"""GPU parity tests for fused_chunk_retention (plain retention), through the C ABI.
+
+Bar (helpers.assert_close): rtol = 2e-2, atol = 2e-2 * max(1, RMS(ref)), RMS error ratio < 0.005,
+against the fp32 oracle evaluated on the same bf16-rounded, seeded inputs."""
+import pytest
+import torch
+
+import helpers as hp
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, oracle_batches=None):
+    """fwd + bwd through the autograd Function; oracle on `oracle_batches` (default: all)."""
+    from flash_pop_amd import fused_chunk_retention
+    _say(f"[plain] B{B} T{T} H{H} dk{dk} dv{dv} s0={state_std} seed={seed}")
+    decays = oracle.head_decays(H, decay_range)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=seed, state_std=state_std)
+    d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=seed + 1)
+    leaves = [None if t is None else t.to(DEV).requires_grad_() for t in (q, k, v, s)]
+    o, S = fused_chunk_retention(*leaves, decays)
+    assert o.dtype == torch.bfloat16 and o.is_contiguous() and S.shape == (B, H, dk, dv)
+    torch.autograd.backward([o, S], [d_o.to(DEV), d_s.to(DEV) if with_ds else torch.zeros_like(S)])
+    torch.cuda.synchronize()
+    bsel = list(range(B)) if oracle_batches is None else oracle_batches
+    for b in bsel:
+        sl = slice(b, b + 1)
+        o_ref, S_ref, grads = hp.oracle_plain(q[sl], k[sl], v[sl], None if s is None else s[sl], decays, d_o[sl],
+                                              d_s[sl] if with_ds else None)
+        hp.assert_close(o[sl], o_ref, f"o[b={b}]")
+        hp.assert_close(S[sl], S_ref, f"S[b={b}]")
+        for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), leaves, grads):
+            if ref is not None:
+                hp.assert_close(leaf.grad[sl], ref, f"{name}[b={b}]")
+    return o, S, [None if l is None else l.grad for l in leaves]
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,state_std", [
+    (2, 256, 4, 64, 64, 0.0),        # reference fwd test family (tests/test_fused_retention.py:184-214)
+    (3, 400, 4, 64, 128, 0.0),       # T not a multiple of the chunk
+    (2, 200, 4, 128, 128, 0.1),      # headline head dims, ragged, carried state
+    (1, 64, 2, 128, 64, None),       # exactly one chunk, no state argument
+    (2, 37, 3, 64, 64, 0.5),         # shorter than one chunk
+    (1, 1, 2, 64, 64, 0.5),          # single token
+    (1, 300, 2, 128, 256, 0.02),     # config-3 head dims
+    (1, 130, 2, 256, 128, 0.1),      # dk = 256
+    (2, 2048, 4, 64, 128, 0.0),      # reference grads test shape (tests/test_fused_retention.py:240-282)
+])
+def test_parity_sweep(B, T, H, dk, dv, state_std):
+    run_plain(B, T, H, dk, dv, state_std, seed=T + dk)
+
+
+def test_decay_range_of_reference_tests():
+    # decays 1 - 2^-linspace(5, 12, H) (tests/test_fused_retention.py:20-25)
+    run_plain(2, 512, 4, 64, 128, 0.0, seed=5, decay_range=(5, 12))
+
+
+def test_config2_headline_shape():
+    """BASELINE config 2 at full size: B8 H16 T4096 d128, zero initial state, dS_final = 0.
+    Oracle on two batch entries (streams are independent); the rest is covered by invariants."""
+    o, S, grads = run_plain(8, 4096, 16, 128, 128, 0.0, seed=0, with_ds=False, oracle_batches=[0, 7])
+    assert all(torch.isfinite(t.float()).all() for t in (o, S, *grads))
+
+
+def test_config3_long_context_carried_state():
+    """BASELINE config 3: B2 H8 T16384 dk128 dv256, S0 ~ N(0, 0.02^2), gradient of the final state too."""
+    run_plain(2, 16384, 8, 128, 256, 0.02, seed=3, with_ds=True, oracle_batches=[1])
+
+
+def test_split_sequence_equals_one_run_at_full_size():
+    """Running [0, T1) then [T1, T) with the carried state must reproduce the single run up to the
+    bf16 rounding of the hand-over state (size-independent property, config-2 shape)."""
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, d = 8, 4096, 16, 128
+    decays = oracle.head_decays(H)
+    q, k, v, _ = hp.make_inputs(B, T, H, d, d, seed=11, device=DEV)
+    o, S = fused_chunk_retention(q, k, v, None, decays)
+    T1 = 1000   # not a chunk multiple on purpose
+    o1, S1 = fused_chunk_retention(q[:, :T1], k[:, :T1], v[:, :T1], None, decays)
+    o2, S2 = fused_chunk_retention(q[:, T1:], k[:, T1:], v[:, T1:], S1, decays)
+    assert torch.equal(o1, o[:, :T1])
+    hp.assert_close(torch.cat((o1, o2), 1), o.float(), "split o")
+    hp.assert_close(S2, S.float(), "split S")
+
+
+def test_linearity_in_v_and_state_at_full_size():
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, d = 8, 4096, 16, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=12, state_std=0.1, device=DEV)
+    o, S = fused_chunk_retention(q, k, v, s, decays)
+    o2, S2 = fused_chunk_retention(q, k, v * 2, s * 2, decays)      # powers of two are exact in bf16
+    assert torch.equal(o2.float(), o.float() * 2) and torch.equal(S2.float(), S.float() * 2)
+
+
+def test_bitwise_reproducible():
+    B, T, H, d = 2, 1000, 4, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=13, state_std=0.1, device=DEV)
+    d_o, d_s = hp.make_cotangents([(B, T, H, d), (B, H, d, d)], seed=14, device=DEV)
+    from flash_pop_amd import _lib
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    a = hp.raw_fwd(lib, q, k, v, s, decays, stream) + hp.raw_bwd(lib, q, k, v, s, decays, d_o, d_s, stream)
+    b = hp.raw_fwd(lib, q, k, v, s, decays, stream) + hp.raw_bwd(lib, q, k, v, s, decays, d_o, d_s, stream)
+    torch.cuda.synchronize()
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_non_contiguous_inputs_and_side_stream():
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, d = 2, 130, 2, 64
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=15, state_std=0.1, device=DEV)
+    o, S = fused_chunk_retention(q, k, v, s, decays)
+    # head-major storage viewed as [B,T,H,d]
+    qt, kt, vt = (x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for x in (q, k, v))
+    assert not qt.is_contiguous()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        o2, S2 = fused_chunk_retention(qt, kt, vt, s, decays)
+    side.synchronize()
+    assert torch.equal(o, o2) and torch.equal(S, S2)
+
+
+def test_state_none_equals_zero_state_and_grad_flags():
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, d = 1, 100, 2, 64
+    decays = oracle.head_decays(H)
+    q, k, v, _ = hp.make_inputs(B, T, H, d, d, seed=16, device=DEV)
+    z = torch.zeros(B, H, d, d, dtype=torch.bfloat16, device=DEV)
+    o1, S1 = fused_chunk_retention(q, k, v, None, decays)
+    o2, S2 = fused_chunk_retention(q, k, v, z, decays)
+    assert torch.equal(o1, o2) and torch.equal(S1, S2)
+    # only q requires grad; the state does not
+    ql = q.clone().requires_grad_()
+    o3, _ = fused_chunk_retention(ql, k, v, z, decays)
+    o3.float().sum().backward()
+    assert ql.grad is not None and ql.grad.shape == q.shape
+
+
+def test_recurrent_decode_matches_chunkwise():
+    """Feeding tokens one at a time with the carried state (flash_pop/retnet.py:79-101 semantics)
+    reproduces the chunkwise outputs up to the bf16 rounding of the carried state."""
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, d = 2, 24, 2, 64
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=17, state_std=0.2, device=DEV)
+    o, S = fused_chunk_retention(q, k, v, s, decays)
+    state, outs = s, []
+    for t in range(T):
+        o_t, state = fused_chunk_retention(q[:, t:t + 1], k[:, t:t + 1], v[:, t:t + 1], state, decays)
+        outs.append(o_t)
+    hp.assert_close(torch.cat(outs, 1), o.float(), "decode o", rms_bar=2e-2)
+    hp.assert_close(state, S.float(), "decode S", rms_bar=2e-2)
