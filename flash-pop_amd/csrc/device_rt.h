@@ -33,6 +33,20 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
-FP_DEVICE float exp2_approx(float x) { return exp2f(x); }
+// 2^x for x <= 0 (v_exp_f32, ~1 ulp; results below the normal range flush to zero).
+FP_DEVICE float exp2_approx(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Bounds-checked view of global memory (raw buffer resource): loads beyond `nbytes` return
+// zero and stores beyond it are dropped by the hardware, which is how ragged chunk tails
+// are handled without branches.  Offsets are bytes from `base`, below 4 GiB.
+struct BufView {
+  __amdgpu_buffer_rsrc_t rsrc;
+};
+FP_DEVICE BufView make_buf(const void* base, uint32_t nbytes) {
+  return BufView{__builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)nbytes, 0x00020000)};
+}
+FP_DEVICE u32x4 buf_load128(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, off, 0, 0); }
+FP_DEVICE u32x2 buf_load64(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b64(b.rsrc, off, 0, 0); }
+FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, b.rsrc, off, 0, 0); }
 
 }  // namespace fprt

@@ -47,6 +47,9 @@ int check_shape(const Shape& s, const double* decays) {
   if (!dim_ok(s.dk) || !dim_ok(s.dv))
     return fail(FP_ERR_UNSUPPORTED_DIM, "dk and dv must be 64, 128 or 256 (got dk=%d, dv=%d)", s.dk, s.dv);
   // per-tensor element counts are indexed with size_t in the kernel; the grid is an int
+  // the kernels address one (batch, head) stream with 32-bit byte offsets
+  const long long span = 2LL * s.T * s.H * (s.dk > s.dv ? s.dk : s.dv);
+  if (span >= (1LL << 32)) return fail(FP_ERR_BAD_SHAPE, "T * H * max(dk, dv) too large: one sequence must stay below 4 GiB");
   const long long wgs = (long long)s.B * s.H * ((s.dk > s.dv ? s.dk : s.dv) / fpk::BV);
   if (wgs > 0x7fffffffLL) return fail(FP_ERR_BAD_SHAPE, "B * H too large");
   for (int h = 0; h < s.H; ++h) {

@@ -1,36 +1,44 @@
-// gfx950 entry points of the pass kernel and the launcher the C-ABI layer calls.
+// gfx950 entry points of the pass kernels and the launcher the C-ABI layer calls.
 #include "device_rt.h"
 #include "retention_pass.h"
+#include "retention_pass_ws.h"
 
 namespace {
 
+// dA = 64, 128: wave-specialised, 8 waves, double-buffered LDS.
+template <int DA>
+__global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(const fpk::PassArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::retention_pass_ws<DA>(args, lds);
+}
+
+// dA = 256: 4 symmetric waves, single-buffered LDS (two stages of 256-wide tiles do not fit).
 template <int DA>
 __global__ __launch_bounds__(fpk::NTHREADS) void retention_pass_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   fpk::retention_pass<DA>(args, lds);
 }
 
-template <int DA>
-int launch(const fpk::PassArgs& a, hipStream_t stream, const char** err) {
+template <typename Kernel>
+int launch(Kernel kernel, int threads, int lds, int* armed_device, const fpk::PassArgs& a, hipStream_t stream,
+           const char** err) {
   // LDS above 64 KB has to be opted into, once per device and kernel.
-  static thread_local int armed_device = -1;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     *err = "hipGetDevice failed";
     return 1;
   }
-  constexpr int lds = fpk::lds_bytes(DA);
-  if (armed_device != dev) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_pass_kernel<DA>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+  if (*armed_device != dev) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
+        hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    armed_device = dev;
+    *armed_device = dev;
   }
   const int nwg = a.B * a.H * (a.dB / fpk::BV);
-  hipLaunchKernelGGL(retention_pass_kernel<DA>, dim3(nwg), dim3(fpk::NTHREADS), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     *err = hipGetErrorString(e);
@@ -43,10 +51,14 @@ int launch(const fpk::PassArgs& a, hipStream_t stream, const char** err) {
 
 int fpk_launch_pass(const fpk::PassArgs& a, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
+  static thread_local int armed[3] = {-1, -1, -1};
   switch (a.dA) {
-    case 64: return launch<64>(a, s, err);
-    case 128: return launch<128>(a, s, err);
-    case 256: return launch<256>(a, s, err);
+    case 64:
+      return launch(retention_pass_ws_kernel<64>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
+    case 128:
+      return launch(retention_pass_ws_kernel<128>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[1], a, s, err);
+    case 256:
+      return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[2], a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }

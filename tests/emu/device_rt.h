@@ -76,4 +76,23 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 
 FP_DEVICE float exp2_approx(float x) { return std::exp2(x); }
 
+struct BufView {
+  const char* base;
+  uint32_t nbytes;
+};
+FP_DEVICE BufView make_buf(const void* base, uint32_t nbytes) { return BufView{static_cast<const char*>(base), nbytes}; }
+FP_DEVICE u32x4 buf_load128(BufView b, uint32_t off) {
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if ((uint64_t)off + 16 <= b.nbytes) std::memcpy(&v, b.base + off, 16);
+  return v;
+}
+FP_DEVICE u32x2 buf_load64(BufView b, uint32_t off) {
+  u32x2 v = {0u, 0u};
+  if ((uint64_t)off + 8 <= b.nbytes) std::memcpy(&v, b.base + off, 8);
+  return v;
+}
+FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) {
+  if ((uint64_t)off + 16 <= b.nbytes) std::memcpy(const_cast<char*>(b.base) + off, &v, 16);
+}
+
 }  // namespace fprt

@@ -1,7 +1,8 @@
-// CPU implementation of fpk_launch_pass: runs the kernel body with 256 OS threads per
-// workgroup, workgroups one after another.  Test infrastructure only.
+// CPU implementation of fpk_launch_pass: runs the kernel bodies with one OS thread per GPU
+// lane, workgroups one after another.  Test infrastructure only.
 #include "device_rt.h"
 #include "retention_pass.h"
+#include "retention_pass_ws.h"
 
 #include <thread>
 #include <vector>
@@ -12,17 +13,16 @@ thread_local LaneCtx g_lane;
 
 namespace {
 
-template <int DA>
-int launch(const fpk::PassArgs& a) {
-  const int nwg = a.B * a.H * (a.dB / fpk::BV);
+template <typename Body>
+int run_grid(int nthreads, int nwg, int lds_bytes, Body body) {
   // exactly the bytes the GPU launch reserves, on the heap so that ASan sees overruns
-  std::vector<char>* lds = new std::vector<char>(fpk::lds_bytes(DA));
+  std::vector<char>* lds = new std::vector<char>(lds_bytes);
   pthread_barrier_t wg_bar;
-  pthread_barrier_init(&wg_bar, nullptr, fpk::NTHREADS);
-  std::vector<fprt::WaveShared> waves(fpk::NTHREADS / 64);
+  pthread_barrier_init(&wg_bar, nullptr, nthreads);
+  std::vector<fprt::WaveShared> waves(nthreads / 64);
   for (auto& w : waves) pthread_barrier_init(&w.bar, nullptr, 64);
   std::vector<std::thread> lanes;
-  for (int t = 0; t < fpk::NTHREADS; ++t) {
+  for (int t = 0; t < nthreads; ++t) {
     lanes.emplace_back([&, t] {
       fprt::g_lane.tid = t;
       fprt::g_lane.grid = nwg;
@@ -30,7 +30,7 @@ int launch(const fpk::PassArgs& a) {
       fprt::g_lane.wg_bar = &wg_bar;
       for (int wg = 0; wg < nwg; ++wg) {
         fprt::g_lane.block = wg;
-        fpk::retention_pass<DA>(a, lds->data());
+        body(lds->data());
         pthread_barrier_wait(&wg_bar);
       }
     });
@@ -45,10 +45,14 @@ int launch(const fpk::PassArgs& a) {
 }  // namespace
 
 int fpk_launch_pass(const fpk::PassArgs& a, void* /*stream*/, const char** err) {
+  const int nwg = a.B * a.H * (a.dB / fpk::BV);
   switch (a.dA) {
-    case 64: return launch<64>(a);
-    case 128: return launch<128>(a);
-    case 256: return launch<256>(a);
+    case 64:
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64>(a, l); });
+    case 128:
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128>(a, l); });
+    case 256:
+      return run_grid(fpk::NTHREADS, nwg, fpk::lds_bytes(256), [&](char* l) { fpk::retention_pass<256>(a, l); });
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }
