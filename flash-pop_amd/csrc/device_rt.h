@@ -36,6 +36,9 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 // 2^x for x <= 0 (v_exp_f32, ~1 ulp; results below the normal range flush to zero).
 FP_DEVICE float exp2_approx(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Nothing may be moved across this point by the instruction scheduler.
+FP_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+
 // Bounds-checked view of global memory (raw buffer resource): loads beyond `nbytes` return
 // zero and stores beyond it are dropped by the hardware, which is how ragged chunk tails
 // are handled without branches.  Offsets are bytes from `base`, below 4 GiB.
@@ -48,5 +51,27 @@ FP_DEVICE BufView make_buf(const void* base, uint32_t nbytes) {
 FP_DEVICE u32x4 buf_load128(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, off, 0, 0); }
 FP_DEVICE u32x2 buf_load64(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b64(b.rsrc, off, 0, 0); }
 FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, b.rsrc, off, 0, 0); }
+
+// Optional instrumentation for profiling builds only.
+//   -DFPK_DBGFLAGS : run-time switches that disable parts of the kernel (timing experiments)
+//   -DFPK_PROFILE  : timeline stamps; slot k of iteration `it` records the shader clock for
+//                    lane 0 of the calling wave of workgroup 0 (perturbs the timing noticeably)
+#ifdef FPK_DBGFLAGS
+__device__ int g_dbg_flags = 0;   // 1 no global loads, 2 readout waves idle, 4 state waves idle
+FP_DEVICE int dbg_flags() { return g_dbg_flags; }
+#else
+FP_DEVICE int dbg_flags() { return 0; }
+#endif
+#ifdef FPK_PROFILE
+__device__ unsigned long long* g_prof_buf = nullptr;
+FP_DEVICE void prof_stamp(int it, int slot) {
+  if (g_prof_buf && blockIdx.x == 0 && (threadIdx.x & 63) == 0 && it < 64) {
+    const int wave = threadIdx.x >> 6;
+    g_prof_buf[(wave * 64 + it) * 8 + slot] = __builtin_amdgcn_s_memtime();
+  }
+}
+#else
+FP_DEVICE void prof_stamp(int, int) {}
+#endif
 
 }  // namespace fprt

@@ -49,6 +49,17 @@ int launch(Kernel kernel, int threads, int lds, int* armed_device, const fpk::Pa
 
 }  // namespace
 
+#ifdef FPK_PROFILE
+extern "C" int fpk_prof_set(void* buf) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fprt::g_prof_buf), &buf, sizeof buf);
+}
+#endif
+#ifdef FPK_DBGFLAGS
+extern "C" int fpk_dbg_set(int flags) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fprt::g_dbg_flags), &flags, sizeof flags);
+}
+#endif
+
 int fpk_launch_pass(const fpk::PassArgs& a, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   static thread_local int armed[3] = {-1, -1, -1};

@@ -6,7 +6,9 @@
 //
 //   readout waves (0..3)  scores^T = W X^T -> P (bf16, in registers) ; Y^T = wread (R X^T) + Z^T P^T
 //                         -> Y tile into LDS.  2 x 2 grid: `ib` = 32 chunk rows, `nb` = 32 columns.
-//   state waves   (4..7)  all global traffic (bounds-checked buffer loads one chunk ahead in
+//                         Branch-free: every wave computes both 32 x 32 score tiles of its rows;
+//                         the tile outside the decay window is cleared after conversion.
+//   state waves   (4..7)  all global traffic (bounds-checked buffer loads two chunks ahead in
 //                         registers, Y tile stores), the transposes of W and Z into LDS, the
 //                         state update R = gamma^L R + (wkey W)^T Z in fp32 accumulators and its
 //                         bf16 copy for the read-out.
@@ -15,6 +17,10 @@
 // state waves finish chunk i's state update and fill stage (i + 1) & 1 with chunk i + 1.  One
 // workgroup barrier per chunk.  The weighted, transposed W tile is private to the state wave
 // that both writes and reads it, so it needs no second buffer and no barrier.
+//
+// Within a chunk the code is laid out in phases separated by scheduling fences: all LDS
+// operands of a phase are requested first, the MFMAs that consume them follow back to back,
+// and the vector work of one phase sits in the shadow of the next phase's MFMAs.
 #pragma once
 #include "pass_args.h"
 #include "retention_pass.h"   // ld/st helpers, acc_row
@@ -29,6 +35,12 @@ constexpr int lds_bytes_ws(int dA) {
               + 2 * BV * (dA + 8)      // bf16 copy of R (transposed), two stages
               + 2 * CH * (BV + 8)      // Y staging, two stages
               + 4 * 32 * (CH + 4));    // weighted W transposed, one 32-row slab per state wave
+}
+
+// two 8-byte LDS reads that form one MFMA operand: tokens 16 kt + 4 g + {0..3} and + 8
+FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
+  const u32x2 lo = ld64(p), hi = ld64(p + 8);
+  return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
 template <int DA>
@@ -64,6 +76,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const int bh = wg / ntile;
   const int h = bh % p.H, b = bh / p.H;
 
+  const int dbg = fprt::dbg_flags();   // always 0 outside profiling builds
   const int T = p.T, bs = p.block;
   const bool rev = p.reverse != 0;
   const float lg = p.log2g[h];
@@ -97,21 +110,34 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   if (!state_role) {
     // =============================== readout waves ===============================
     const int ib = wave >> 1, nb = wave & 1;
-    float mw_diag[16], mw_off[16];
+    // Of the two 32-token score tiles of this wave's rows, the "diagonal" one (tokens 32 ib ..)
+    // is half masked; the "other" one (tokens 32 (1 - ib) ..) lies either wholly inside the
+    // decay window or wholly outside it.  Masked scores are zeroed by clearing their bits after
+    // the bf16 conversion, so that inf or nan in a masked operand cannot leak through 0 * x.
+    const bool other_live = rev ? (ib == 0) : (ib == 1);
+    float mw_d[16], mw_o[16];
+    uint32_t keep_d[8];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int jl = acc_row(r, g);
-      const int d = rev ? (jl - c) : (c - jl);
-      mw_diag[r] = d >= 0 ? p.s_intra * fprt::exp2_approx((float)d * lg) : 0.f;
-      mw_off[r] = p.s_intra * fprt::exp2_approx((float)(32 + d) * lg);
+      const int d = rev ? (jl - c) : (c - jl);          // distance inside the diagonal tile
+      mw_d[r] = p.s_intra * fprt::exp2_approx((float)(d >= 0 ? d : 0) * lg);
+      mw_o[r] = p.s_intra * fprt::exp2_approx((float)(32 + d) * lg);
     }
-    const bool need_off = rev ? (ib == 0) : (ib == 1);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d0 = rev ? (acc_row(2 * e, g) - c) : (c - acc_row(2 * e, g));
+      const int d1 = rev ? (acc_row(2 * e + 1, g) - c) : (c - acc_row(2 * e + 1, g));
+      keep_d[e] = (d0 >= 0 ? 0x0000ffffu : 0u) | (d1 >= 0 ? 0xffff0000u : 0u);
+    }
+    const uint32_t keep_o = other_live ? 0xffffffffu : 0u;
     const int i_row = 32 * ib + c;                 // this lane's chunk row (query index)
     const int x_off = i_row * X_LD + 8 * g;
     const int wd_off = (32 * ib + c) * X_LD + 8 * g;
     const int wo_off = (32 * (1 - ib) + c) * X_LD + 8 * g;
     const int r_off = (32 * nb + c) * RT_LD + 8 * g;
-    const int z_off = (32 * nb + c) * T_LD + 4 * g;
+    const int zd_off = (32 * nb + c) * T_LD + 4 * g + 32 * ib;
+    const int zo_off = (32 * nb + c) * T_LD + 4 * g + 32 * (1 - ib);
     const int y_off = i_row * YB_LD + 32 * nb + 4 * g;
     const float wread_fwd = p.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
 
@@ -131,58 +157,81 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         wread = p.s_read * fprt::exp2_approx((float)e * lg);
       }
 
-      u32x4 xf[KS];
+      fprt::prof_stamp(it, 0);
+      if (dbg & 2) {
+        fprt::block_sync();
+        const int pos = next_pos(t0, L);
+        if (!has_more(pos)) break;
+        chunk_at(pos, t0, L);
+        continue;
+      }
+      // ---- phase 0: request X, R and the diagonal W tile
+      u32x4 xf[KS], rf[KS], wd[KS], wo[KS], zd[2], zo[2];
 #pragma unroll
-      for (int t = 0; t < KS; ++t) xf[t] = ld128(xs + x_off + 16 * t);
+      for (int t = 0; t < KS; ++t) {
+        xf[t] = ld128(xs + x_off + 16 * t);
+        rf[t] = ld128(rt + r_off + 16 * t);
+      }
+#pragma unroll
+      for (int t = 0; t < KS; ++t) wd[t] = ld128(ws + wd_off + 16 * t);
+      fprt::sched_fence();
 
-      // read-out of the carried state: Y^T[n][i] = sum_a R[a][n] X[i][a]
+      // ---- phase 1: read-out of the carried state, Y^T[n][i] = sum_a R[a][n] X[i][a]
       f32x16 yacc = {0};
 #pragma unroll
-      for (int t = 0; t < KS; ++t) yacc = fprt::mfma_32x32x16_bf16(ld128(rt + r_off + 16 * t), xf[t], yacc);
+      for (int t = 0; t < KS; ++t) yacc = fprt::mfma_32x32x16_bf16(rf[t], xf[t], yacc);
+      fprt::sched_fence();
+      fprt::prof_stamp(it, 1);
 
-      // scores^T tiles -> P fragments
-      u32x4 pf_diag[2], pf_off[2];
-      {
-        f32x16 sc = {0};
+      // ---- phase 2: scores^T of the diagonal tile; the other W tile and Z arrive meanwhile (the
+      // W tile takes over the registers of the R fragments)
 #pragma unroll
-        for (int t = 0; t < KS; ++t) sc = fprt::mfma_32x32x16_bf16(ld128(ws + wd_off + 16 * t), xf[t], sc);
+      for (int t = 0; t < KS; ++t) wo[t] = ld128(ws + wo_off + 16 * t);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            pf_diag[t][e] = fprt::pack_bf16x2(sc[8 * t + 2 * e] * mw_diag[8 * t + 2 * e],
-                                              sc[8 * t + 2 * e + 1] * mw_diag[8 * t + 2 * e + 1]);
-          }
-        }
+      for (int t = 0; t < 2; ++t) {
+        zd[t] = ld_token_frag(zt + zd_off + 16 * t);
+        zo[t] = ld_token_frag(zt + zo_off + 16 * t);
       }
-      if (need_off) {
-        f32x16 sc = {0};
+      f32x16 sd = {0};
 #pragma unroll
-        for (int t = 0; t < KS; ++t) sc = fprt::mfma_32x32x16_bf16(ld128(ws + wo_off + 16 * t), xf[t], sc);
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            pf_off[t][e] = fprt::pack_bf16x2(sc[8 * t + 2 * e] * mw_off[8 * t + 2 * e],
-                                             sc[8 * t + 2 * e + 1] * mw_off[8 * t + 2 * e + 1]);
-          }
-        }
-      }
+      for (int t = 0; t < KS; ++t) sd = fprt::mfma_32x32x16_bf16(wd[t], xf[t], sd);
+      fprt::sched_fence();
+      fprt::prof_stamp(it, 2);
 
+      // ---- phase 3: scores^T of the other tile; the read-out is scaled and P of the diagonal
+      // tile converted in its shadow.  Accumulator element r = 8 t + e is token
+      // 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the order the Z fragments are read in.
+      f32x16 so = {0};
+#pragma unroll
+      for (int t = 0; t < KS; ++t) so = fprt::mfma_32x32x16_bf16(wo[t], xf[t], so);
 #pragma unroll
       for (int r = 0; r < 16; ++r) yacc[r] *= wread;
-
-      // Y^T += Z^T P^T ; k-step kt covers tokens 16 kt .. 16 kt + 15 in the order P holds them
-      auto zfrag = [&](int kt) {
-        const u32x2 lo = ld64(zt + z_off + 16 * kt), hi = ld64(zt + z_off + 16 * kt + 8);
-        return u32x4{lo[0], lo[1], hi[0], hi[1]};
-      };
+      u32x4 pd[2], po[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zfrag(2 * ib + t), pf_diag[t], yacc);
-      if (need_off) {
+      for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zfrag(2 * (1 - ib) + t), pf_off[t], yacc);
+        for (int e = 0; e < 4; ++e) {
+          const int r = 8 * t + 2 * e;
+          pd[t][e] = fprt::pack_bf16x2(sd[r] * mw_d[r], sd[r + 1] * mw_d[r + 1]) & keep_d[4 * t + e];
+        }
       }
+      fprt::sched_fence();
+      fprt::prof_stamp(it, 3);
+
+      // ---- phase 4: Y^T += Z^T P^T
+#pragma unroll
+      for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zd[t], pd[t], yacc);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 8 * t + 2 * e;
+          po[t][e] = fprt::pack_bf16x2(so[r] * mw_o[r], so[r + 1] * mw_o[r + 1]) & keep_o;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zo[t], po[t], yacc);
+      fprt::sched_fence();
 
       // accumulator element r holds column n = 32 nb + 8 (r / 4) + 4 g + r % 4 of row i_row
 #pragma unroll
@@ -192,8 +241,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         d[1] = fprt::pack_bf16x2(yacc[4 * qd + 2], yacc[4 * qd + 3]);
         st64(yb + y_off + 8 * qd, d);
       }
+      fprt::prof_stamp(it, 4);
 
       fprt::block_sync();
+      fprt::prof_stamp(it, 5);
       const int pos = next_pos(t0, L);
       if (!has_more(pos)) break;
       chunk_at(pos, t0, L);
@@ -212,13 +263,13 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const uint32_t rowA = (uint32_t)p.H * p.dA * 2, rowB = (uint32_t)p.H * p.dB * 2;   // bytes
   const size_t streamA = ((size_t)b * T * p.H + h) * p.dA;
   const size_t streamB = ((size_t)b * T * p.H + h) * p.dB + (size_t)tile * BV;
-  const uint16_t* const Xg = p.X + streamA;
-  const uint16_t* const Wg = p.W + streamA;
-  const uint16_t* const Zg = p.Z + streamB;
-  uint16_t* const Yg = p.Y + streamB;
+  const char* const Xg = reinterpret_cast<const char*>(p.X + streamA);
+  const char* const Wg = reinterpret_cast<const char*>(p.W + streamA);
+  const char* const Zg = reinterpret_cast<const char*>(p.Z + streamB);
+  char* const Yg = reinterpret_cast<char*>(p.Y + streamB);
   const size_t mat = (size_t)p.dA * p.dB;
 
-  // per-thread load coordinates (bytes relative to the chunk's first row)
+  // per-thread coordinates, bytes relative to the chunk's first row; they never change
   uint32_t xg_off[NXP];
   int xs_off[NXP];
 #pragma unroll
@@ -228,28 +279,40 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     xs_off[u] = row * X_LD + col * 8;
   }
   const int w_fg = lane & 3, w_tg = lane >> 2;       // W unit: tokens 4 w_tg.., features 32 ablk + 8 w_fg..
-  const uint32_t wg_off = (4 * w_tg) * rowA + (32 * ablk + 8 * w_fg) * 2;
+  uint32_t wg_off[4], zg_off[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) wg_off[r] = (4 * w_tg + r) * rowA + (32 * ablk + 8 * w_fg) * 2;
   const int ws_off = (4 * w_tg) * X_LD + 32 * ablk + 8 * w_fg;
   const int wt_off = (8 * w_fg) * T_LD + 4 * w_tg;
   const int z_tg = rt_id >> 4, z_fq = rt_id & 15;    // Z unit: tokens 4 z_tg.., columns 4 z_fq..
-  const uint32_t zg_off = (4 * z_tg) * rowB + z_fq * 8;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) zg_off[r] = (4 * z_tg + r) * rowB + z_fq * 8;
   const int zt_off = (4 * z_fq) * T_LD + 4 * z_tg;
   const int y_row = rt_id >> 2, y_col = (rt_id & 3) * 16;
+  const uint32_t yg_off = y_row * rowB + y_col * 2;
 
-  u32x4 px[NXP], pw[4];
-  u32x2 pz[4];
-  auto prefetch = [&](int ct0, int cL) {
-    // bytes from the stream base up to the end of the chunk's last row: later rows read as zero
-    const uint32_t endA = (uint32_t)(ct0 + cL - 1) * rowA + p.dA * 2;
-    const uint32_t endB = (uint32_t)(ct0 + cL - 1) * rowB + BV * 2;
-    const fprt::BufView xb = fprt::make_buf(Xg, endA), wb = fprt::make_buf(Wg, endA), zb = fprt::make_buf(Zg, endB);
-    const uint32_t baseA = (uint32_t)ct0 * rowA, baseB = (uint32_t)ct0 * rowB;
+  // Two register sets of loaded chunks, so that global loads run two chunks ahead of the math.
+  struct ChunkRegs {
+    u32x4 x[NXP], w[4];
+    u32x2 z[4];
+  };
+  ChunkRegs setA, setB;
+  // Loads are issued unconditionally so that the number of outstanding memory operations is the
+  // same in every iteration; a chunk that does not exist gets zero-length views (no traffic).
+  auto prefetch = [&](ChunkRegs& cr, int ct0, int cL, bool ok) {
+    // views that start at the chunk's first row and end with its last: later rows read as zero
+    const bool live = ok && !(dbg & 1);
+    const uint32_t lenA = live ? (uint32_t)(cL - 1) * rowA + p.dA * 2 : 0u;
+    const uint32_t lenB = live ? (uint32_t)(cL - 1) * rowB + BV * 2 : 0u;
+    const size_t baseA = (size_t)ct0 * rowA, baseB = (size_t)ct0 * rowB;
+    const fprt::BufView xb = fprt::make_buf(Xg + baseA, lenA), wb = fprt::make_buf(Wg + baseA, lenA),
+                        zb = fprt::make_buf(Zg + baseB, lenB);
 #pragma unroll
-    for (int u = 0; u < NXP; ++u) px[u] = fprt::buf_load128(xb, baseA + xg_off[u]);
+    for (int u = 0; u < NXP; ++u) cr.x[u] = fprt::buf_load128(xb, xg_off[u]);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) pw[r] = fprt::buf_load128(wb, baseA + wg_off + r * rowA);
+    for (int r = 0; r < 4; ++r) cr.w[r] = fprt::buf_load128(wb, wg_off[r]);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) pz[r] = fprt::buf_load64(zb, baseB + zg_off + r * rowB);
+    for (int r = 0; r < 4; ++r) cr.z[r] = fprt::buf_load64(zb, zg_off[r]);
   };
 
   // state tiles: racc[nn] is R[32 ablk + acc_row][32 (nb0 + nn) + c]
@@ -276,23 +339,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     }
   };
 
-  // registers (chunk of length cL) + R -> LDS stage s
-  int Lk_cached = -1;
-  float wkey[4];
-  auto fill_stage = [&](int s, int cL) {
-    if (cL != Lk_cached) {
-      Lk_cached = cL;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int j = 4 * w_tg + r;
-        int e = rev ? (j + 1) : (cL - 1 - j);
-        if (e < 0) e = 0;
-        wkey[r] = p.s_update * fprt::exp2_approx((float)e * lg);
-      }
-    }
-    uint16_t* xs = XS + s * CH * X_LD;
-    uint16_t* ws = WS + s * CH * X_LD;
-    uint16_t* zt = ZT + s * BV * T_LD;
+  // bf16 copy of R -> LDS stage s
+  auto write_rt = [&](int s) {
     uint16_t* rt = RT + s * BV * RT_LD;
 #pragma unroll
     for (int nn = 0; nn < NNW; ++nn) {
@@ -304,17 +352,29 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         st64(rt + (32 * (nb0 + nn) + c) * RT_LD + 32 * ablk + 8 * qd + 4 * g, d);
       }
     }
+  };
+
+  // A loaded chunk of length cL goes to LDS stage s: the weighted W^T slab and Z^T are formed in
+  // registers and written at once (short live ranges), the row-major X and W tiles are copies.
+  int Lk_cached = -1;
+  float wkey[4];
+  auto store_transposed = [&](const ChunkRegs& cr, int s, int cL) {
+    if (cL != Lk_cached) {
+      Lk_cached = cL;
 #pragma unroll
-    for (int u = 0; u < NXP; ++u) st128(xs + xs_off[u], px[u]);
-    if (ws_writer) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) st128(ws + ws_off + r * X_LD, pw[r]);
+      for (int r = 0; r < 4; ++r) {
+        const int j = 4 * w_tg + r;
+        int e = rev ? (j + 1) : (cL - 1 - j);
+        if (e < 0) e = 0;
+        wkey[r] = p.s_update * fprt::exp2_approx((float)e * lg);
+      }
     }
+    uint16_t* zt = ZT + s * BV * T_LD;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       u32x2 d;
-      d[0] = fprt::pack_bf16x2(bf16_elem(pw[0], e) * wkey[0], bf16_elem(pw[1], e) * wkey[1]);
-      d[1] = fprt::pack_bf16x2(bf16_elem(pw[2], e) * wkey[2], bf16_elem(pw[3], e) * wkey[3]);
+      d[0] = fprt::pack_bf16x2(bf16_elem(cr.w[0], e) * wkey[0], bf16_elem(cr.w[1], e) * wkey[1]);
+      d[1] = fprt::pack_bf16x2(bf16_elem(cr.w[2], e) * wkey[2], bf16_elem(cr.w[3], e) * wkey[3]);
       st64(wt + wt_off + e * T_LD, d);
     }
 #pragma unroll
@@ -322,98 +382,168 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       const int w = e >> 1;
       u32x2 d;
       if (e & 1) {
-        d[0] = (pz[0][w] >> 16) | (pz[1][w] & 0xffff0000u);
-        d[1] = (pz[2][w] >> 16) | (pz[3][w] & 0xffff0000u);
+        d[0] = (cr.z[0][w] >> 16) | (cr.z[1][w] & 0xffff0000u);
+        d[1] = (cr.z[2][w] >> 16) | (cr.z[3][w] & 0xffff0000u);
       } else {
-        d[0] = (pz[0][w] & 0xffffu) | (pz[1][w] << 16);
-        d[1] = (pz[2][w] & 0xffffu) | (pz[3][w] << 16);
+        d[0] = (cr.z[0][w] & 0xffffu) | (cr.z[1][w] << 16);
+        d[1] = (cr.z[2][w] & 0xffffu) | (cr.z[3][w] << 16);
       }
       st64(zt + zt_off + e * T_LD, d);
     }
   };
-
-  // Y tile of chunk [ct0, ct0 + cL) from LDS stage s to global; rows beyond cL are dropped
-  auto store_y = [&](int s, int ct0, int cL) {
-    const uint32_t endB = (uint32_t)(ct0 + cL - 1) * rowB + BV * 2;
-    const fprt::BufView yv = fprt::make_buf(Yg, endB);
-    const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
-    const uint32_t off = (uint32_t)(ct0 + y_row) * rowB + y_col * 2;
-    fprt::buf_store128(yv, off, ld128(src));
-    fprt::buf_store128(yv, off + 16, ld128(src + 8));
+  auto store_rowmajor = [&](const ChunkRegs& cr, int s) {
+    uint16_t* xs = XS + s * CH * X_LD;
+    uint16_t* ws = WS + s * CH * X_LD;
+#pragma unroll
+    for (int u = 0; u < NXP; ++u) st128(xs + xs_off[u], cr.x[u]);
+    if (ws_writer) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) st128(ws + ws_off + r * X_LD, cr.w[r]);
+    }
   };
 
-  // ---- prologue: chunk 0 into stage 0, chunk 1 into registers ------------------------
-  prefetch(t0, L);
-  inject(t0 + L);
-  fill_stage(0, L);
-  int t0n = 0, Ln = 0;
-  bool more = has_more(next_pos(t0, L));
-  if (more) {
-    chunk_at(next_pos(t0, L), t0n, Ln);
-    prefetch(t0n, Ln);
-  }
-  fprt::block_sync();
-
-  int t0p = 0, Lp = 0;   // previous chunk, whose Y tile is still in LDS
-  int Lg_cached = -1;
-  float gL = 1.f;
-  for (int it = 0;; ++it) {
-    const int s = it & 1;
-    if (it > 0) store_y(s ^ 1, t0p, Lp);
-
-    // R = gamma^L R + (wkey W)^T Z for chunk `it`
-    if (L != Lg_cached) {
-      Lg_cached = L;
-      gL = fprt::exp2_approx((float)L * lg);
-    }
-    const uint16_t* zt = ZT + s * BV * T_LD;
-#pragma unroll
-    for (int nn = 0; nn < NNW; ++nn) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) racc[nn][r] *= gL;
-    }
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      const uint16_t* wp = wt + c * T_LD + 16 * kt + 4 * g;
-      const u32x2 wlo = ld64(wp), whi = ld64(wp + 8);
-      const u32x4 wf = {wlo[0], wlo[1], whi[0], whi[1]};
-#pragma unroll
-      for (int nn = 0; nn < NNW; ++nn) {
-        const uint16_t* zp = zt + (32 * (nb0 + nn) + c) * T_LD + 16 * kt + 4 * g;
-        const u32x2 zlo = ld64(zp), zhi = ld64(zp + 8);
-        racc[nn] = fprt::mfma_32x32x16_bf16(wf, u32x4{zlo[0], zlo[1], zhi[0], zhi[1]}, racc[nn]);
+  // ---- prologue: chunk 0 into stage 0, chunk 1 in flight ----------------------------------
+  struct Chunk {
+    int t0, L;
+    bool ok;
+  };
+  auto chunk_after = [&](const Chunk& ck) {
+    Chunk n = {0, 0, false};
+    if (ck.ok) {
+      const int pos = next_pos(ck.t0, ck.L);
+      if (has_more(pos)) {
+        n.ok = true;
+        chunk_at(pos, n.t0, n.L);
       }
     }
+    return n;
+  };
+  Chunk cur = {t0, L, true}, nxt = chunk_after(cur), prev = {0, 0, false};
+  prefetch(setA, cur.t0, cur.L, true);
+  prefetch(setB, nxt.t0, nxt.L, nxt.ok);
+  inject(cur.t0 + cur.L);
+  write_rt(0);
+  store_transposed(setA, 0, cur.L);
+  store_rowmajor(setA, 0);
+  fprt::block_sync();
+
+  int Lg_cached = -1;
+  float gL = 1.f;
+  // One iteration: `refill` is the register set freed by the previous iteration (it receives
+  // chunk it + 2), `ready` holds chunk it + 1.  Returns false after the last chunk.
+  auto iteration = [&](int it, ChunkRegs& refill, const ChunkRegs& ready) -> bool {
+    const int s = it & 1;
+    fprt::prof_stamp(it, 0);
+    const Chunk nn = chunk_after(nxt);
+    prefetch(refill, nn.t0, nn.L, nn.ok);
+
+    if (dbg & 4) {
+      fprt::block_sync();
+      if (!nxt.ok) return false;
+      prev = cur;
+      cur = nxt;
+      nxt = nn;
+      return true;
+    }
+    // ---- phase 0: request the operands of the state update (this wave's whole W^T slab, the
+    // first half of Z^T) and the finished Y tile; decay R while they arrive
+    if (cur.L != Lg_cached) {
+      Lg_cached = cur.L;
+      gL = fprt::exp2_approx((float)cur.L * lg);
+    }
+    const uint16_t* zt = ZT + s * BV * T_LD;
+    u32x4 wf[4], zlo[NNW][2], zhi[NNW][2], yv[2];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) wf[kt] = ld_token_frag(wt + c * T_LD + 16 * kt + 4 * g);
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq) zlo[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * kt + 4 * g);
+    }
+    {
+      const uint16_t* src = YB + (s ^ 1) * CH * YB_LD + y_row * YB_LD + y_col;
+      yv[0] = ld128(src);
+      yv[1] = ld128(src + 8);
+    }
+#pragma unroll
+    for (int nq = 0; nq < NNW; ++nq) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) racc[nq][r] *= gL;
+    }
+    fprt::sched_fence();
+    fprt::prof_stamp(it, 1);
+
+    // ---- phase 1: first half of R = gamma^L R + (wkey W)^T Z; in its shadow the rest of Z^T is
+    // requested, the previous Y tile leaves, and chunk it + 1 (zeros if there is none) is
+    // transposed into the other stage.  The W^T slab is overwritten only after all of it was read.
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[kt], zlo[nq][kt], racc[nq]);
+    }
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq)
+        zhi[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * (2 + kt) + 4 * g);
+    }
+    {
+      // rows beyond the chunk's length fall outside the view and are dropped; before the first
+      // chunk the view is empty
+      const fprt::BufView yview =
+          fprt::make_buf(Yg + (size_t)prev.t0 * rowB, prev.ok ? (uint32_t)(prev.L - 1) * rowB + BV * 2 : 0u);
+      fprt::buf_store128(yview, yg_off, yv[0]);
+      fprt::buf_store128(yview, yg_off + 16, yv[1]);
+    }
+    store_transposed(ready, s ^ 1, nxt.L);
+    fprt::sched_fence();
+    fprt::prof_stamp(it, 2);
+
+    // ---- phase 2: second half of the state update; the row-major copies go out in its shadow
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc[nq]);
+    }
+    store_rowmajor(ready, s ^ 1);
+    fprt::sched_fence();
 
     // state after every full block (forward walk)
-    const int t1 = t0 + L;
+    const int t1 = cur.t0 + cur.L;
     if (p.Bout && bs > 0 && (t1 % bs) == 0) {
       uint16_t* dst = p.Bout + (((size_t)b * p.nblk + (t1 / bs - 1)) * p.H + h) * mat;
 #pragma unroll
-      for (int nn = 0; nn < NNW; ++nn) {
+      for (int nq = 0; nq < NNW; ++nq) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dst[state_off(nn, r)] = float_to_bf16_bits(racc[nn][r]);
+        for (int r = 0; r < 16; ++r) dst[state_off(nq, r)] = float_to_bf16_bits(racc[nq][r]);
       }
     }
+    fprt::prof_stamp(it, 3);
 
-    t0p = t0;
-    Lp = L;
-    if (more) {
-      inject(t0n + Ln);
-      fill_stage(s ^ 1, Ln);
-      t0 = t0n;
-      L = Ln;
-      more = has_more(next_pos(t0, L));
-      if (more) {
-        chunk_at(next_pos(t0, L), t0n, Ln);
-        prefetch(t0n, Ln);
-      }
-      fprt::block_sync();
-    } else {
-      fprt::block_sync();
-      store_y(s, t0p, Lp);
-      break;
+    // ---- phase 3: bf16 copy of the new state for the next chunk's read-out
+    if (nxt.ok) {
+      inject(nxt.t0 + nxt.L);
+      write_rt(s ^ 1);
     }
+    fprt::prof_stamp(it, 4);
+    fprt::block_sync();
+    fprt::prof_stamp(it, 5);
+    if (!nxt.ok) {
+      // last Y tile
+      const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
+      const fprt::BufView yview = fprt::make_buf(Yg + (size_t)cur.t0 * rowB, (uint32_t)(cur.L - 1) * rowB + BV * 2);
+      fprt::buf_store128(yview, yg_off, ld128(src));
+      fprt::buf_store128(yview, yg_off + 16, ld128(src + 8));
+      return false;
+    }
+    prev = cur;
+    cur = nxt;
+    nxt = nn;
+    return true;
+  };
+  for (int it = 0;; it += 2) {
+    if (!iteration(it, setA, setB)) break;
+    if (!iteration(it + 1, setB, setA)) break;
   }
 
   if (p.Rout) {

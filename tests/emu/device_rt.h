@@ -76,6 +76,11 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 
 FP_DEVICE float exp2_approx(float x) { return std::exp2(x); }
 
+FP_DEVICE void sched_fence() {}
+
+FP_DEVICE int dbg_flags() { return 0; }
+FP_DEVICE void prof_stamp(int, int) {}
+
 struct BufView {
   const char* base;
   uint32_t nbytes;
