@@ -36,6 +36,10 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 // 2^x for x <= 0 (v_exp_f32, ~1 ulp; results below the normal range flush to zero).
 FP_DEVICE float exp2_approx(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Orders LDS traffic between the lanes of one wave.  The hardware executes a wave's LDS
+// instructions in order, so this only has to stop the compiler from reordering them.
+FP_DEVICE void wave_sync() { __builtin_amdgcn_wave_barrier(); }
+
 // Nothing may be moved across this point by the instruction scheduler.
 FP_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 

@@ -6,10 +6,10 @@
 namespace {
 
 // dA = 64, 128: wave-specialised, 8 waves, double-buffered LDS.
-template <int DA>
+template <int DA, bool BLOCKS>
 __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::retention_pass_ws<DA>(args, lds);
+  fpk::retention_pass_ws<DA, BLOCKS>(args, lds);
 }
 
 // dA = 256: 4 symmetric waves, single-buffered LDS (two stages of 256-wide tiles do not fit).
@@ -62,14 +62,17 @@ extern "C" int fpk_dbg_set(int flags) {
 
 int fpk_launch_pass(const fpk::PassArgs& a, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  static thread_local int armed[3] = {-1, -1, -1};
+  static thread_local int armed[5] = {-1, -1, -1, -1, -1};
+  const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   switch (a.dA) {
     case 64:
-      return launch(retention_pass_ws_kernel<64>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<64, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
+      return launch(retention_pass_ws_kernel<64, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
     case 128:
-      return launch(retention_pass_ws_kernel<128>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[1], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<128, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[2], a, s, err);
+      return launch(retention_pass_ws_kernel<128, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
     case 256:
-      return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[2], a, s, err);
+      return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[4], a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }

@@ -43,7 +43,9 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
   return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
-template <int DA>
+// BLOCKS: the pass writes block states (Bout) or reads their gradients (Bin).  Kept out of the
+// plain instantiation, whose state waves have no registers to spare for it.
+template <int DA, bool BLOCKS>
 FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
   constexpr int X_LD = DA + 8;
@@ -292,6 +294,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const uint32_t yg_off = y_row * rowB + y_col * 2;
 
   // Two register sets of loaded chunks, so that global loads run two chunks ahead of the math.
+  // The block-state instantiation needs the registers of the second set for the block-state
+  // tile in flight and keeps its loads one chunk ahead instead.
+  constexpr bool DEEP = !BLOCKS;
   struct ChunkRegs {
     u32x4 x[NXP], w[4];
     u32x2 z[4];
@@ -317,27 +322,103 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 
   // state tiles: racc[nn] is R[32 ablk + acc_row][32 (nb0 + nn) + c]
   f32x16 racc[NNW];
-  auto state_off = [&](int nn, int r) -> size_t {
-    const int a = 32 * ablk + acc_row(r, g);
-    const size_t n = (size_t)tile * BV + 32 * (nb0 + nn) + c;
-    return (size_t)a * p.rs_a + n * p.rs_n;
+#pragma unroll
+  for (int nn = 0; nn < NNW; ++nn) racc[nn] = f32x16{0};
+
+  // ---- this wave's tile of a state matrix <-> global memory --------------------------------
+  // Global accesses are 16 bytes per lane along the contiguous direction of the matrix; the
+  // change to and from the accumulator layout goes through the part of an R staging buffer that
+  // only this wave writes (rows 32 nb0 .., columns 32 ablk ..), so no barrier is involved.  In
+  // the staging area the tile is kept in the order of the global matrix: for R = S that is
+  // [a][n] (one accumulator element per 2-byte access), for R = S^T it is [n][a], which is also
+  // the natural order of the staging buffer (four accumulator elements per 8-byte access).
+  const bool tposed = p.rs_a == 1;
+  constexpr int NP = 2 * NNW;                    // 16-byte pieces per lane
+  constexpr int NCOL = 32 * NNW;                 // tile columns
+  struct TileRegs {
+    u32x4 v[NP];
   };
+  uint32_t tile_goff[NP];                        // byte offsets inside one state matrix (< 256 KiB)
+  int tile_soff[NP];                             // element offsets inside one staging stage
+  auto stage_elem = [&](int e) { return (32 * nb0 + e / 32) * RT_LD + 32 * ablk + e % 32; };
 #pragma unroll
-  for (int nn = 0; nn < NNW; ++nn) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) racc[nn][r] = p.R0 ? bf16_bits_to_float(p.R0[(size_t)bh * mat + state_off(nn, r)]) : 0.f;
+  for (int u = 0; u < NP; ++u) {
+    const int q = lane + 64 * u;
+    if (!tposed) {
+      const int a_l = q / (4 * NNW), piece = q % (4 * NNW);
+      tile_goff[u] = 2u * (uint32_t)((32 * ablk + a_l) * (int)p.rs_a + tile * BV + 32 * nb0 + 8 * piece);
+      tile_soff[u] = stage_elem(a_l * NCOL + 8 * piece);
+    } else {
+      const int n_l = q / 4, piece = q % 4;
+      tile_goff[u] = 2u * (uint32_t)((tile * BV + 32 * nb0 + n_l) * (int)p.rs_n + 32 * ablk + 8 * piece);
+      tile_soff[u] = stage_elem(n_l * 32 + 8 * piece);
+    }
   }
-  // gradient of the block state that ends at token t1 joins R before that chunk is read out
-  auto inject = [&](int t1) {
-    if (p.Bin && bs > 0 && (t1 % bs) == 0) {
-      const size_t base = (((size_t)b * p.nblk + (t1 / bs - 1)) * p.H + h) * mat;
+  // issue the global loads of a tile; `src` null or !live -> zeros without memory traffic
+  auto tile_load = [&](TileRegs& tr, const uint16_t* src, bool live) {
+    const fprt::BufView view = fprt::make_buf(src, (src && live) ? (uint32_t)(mat * 2) : 0u);
 #pragma unroll
-      for (int nn = 0; nn < NNW; ++nn) {
+    for (int u = 0; u < NP; ++u) tr.v[u] = fprt::buf_load128(view, tile_goff[u]);
+  };
+  // R (+)= loaded tile, through stage s
+  auto tile_accumulate = [&](const TileRegs& tr, int s, bool add) {
+    uint16_t* st = RT + s * BV * RT_LD;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) racc[nn][r] += bf16_bits_to_float(p.Bin[base + state_off(nn, r)]);
+    for (int u = 0; u < NP; ++u) st128(st + tile_soff[u], tr.v[u]);
+    fprt::wave_sync();
+#pragma unroll
+    for (int nn = 0; nn < NNW; ++nn) {
+      if (!tposed) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float x = bf16_bits_to_float(reinterpret_cast<const u16_m*>(st)[stage_elem(acc_row(r, g) * NCOL + 32 * nn + c)]);
+          racc[nn][r] = add ? racc[nn][r] + x : x;
+        }
+      } else {
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const u32x2 d = ld64(st + stage_elem((32 * nn + c) * 32 + 8 * qd + 4 * g));
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const uint32_t w = d[k >> 1];
+            const float x = __builtin_bit_cast(float, (k & 1) ? (w & 0xffff0000u) : (w << 16));
+            racc[nn][4 * qd + k] = add ? racc[nn][4 * qd + k] + x : x;
+          }
+        }
       }
     }
+    fprt::wave_sync();   // the staging area is reused right after
   };
+  // bf16(R) -> global matrix at dst, through stage s
+  auto tile_store = [&](uint16_t* dst, int s) {
+    uint16_t* st = RT + s * BV * RT_LD;
+#pragma unroll
+    for (int nn = 0; nn < NNW; ++nn) {
+      if (!tposed) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          reinterpret_cast<u16_m*>(st)[stage_elem(acc_row(r, g) * NCOL + 32 * nn + c)] = float_to_bf16_bits(racc[nn][r]);
+      } else {
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          u32x2 d;
+          d[0] = fprt::pack_bf16x2(racc[nn][4 * qd], racc[nn][4 * qd + 1]);
+          d[1] = fprt::pack_bf16x2(racc[nn][4 * qd + 2], racc[nn][4 * qd + 3]);
+          st64(st + stage_elem((32 * nn + c) * 32 + 8 * qd + 4 * g), d);
+        }
+      }
+    }
+    fprt::wave_sync();
+    const fprt::BufView view = fprt::make_buf(dst, (uint32_t)(mat * 2));
+#pragma unroll
+    for (int u = 0; u < NP; ++u) fprt::buf_store128(view, tile_goff[u], ld128(st + tile_soff[u]));
+    fprt::wave_sync();   // the staging area is reused right after
+  };
+  // block-state matrix of the block that ends at token t1 (its gradient in a reverse pass)
+  auto block_matrix = [&](const uint16_t* base, int t1) {
+    return base + (((size_t)b * p.nblk + (t1 / bs - 1)) * p.H + h) * mat;
+  };
+  auto ends_block = [&](int t1) { return bs > 0 && (t1 % bs) == 0; };
 
   // bf16 copy of R -> LDS stage s
   auto write_rt = [&](int s) {
@@ -420,11 +501,20 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   };
   Chunk cur = {t0, L, true}, nxt = chunk_after(cur), prev = {0, 0, false};
   prefetch(setA, cur.t0, cur.L, true);
-  prefetch(setB, nxt.t0, nxt.L, nxt.ok);
-  inject(cur.t0 + cur.L);
+  if (DEEP) prefetch(setB, nxt.t0, nxt.L, nxt.ok);
+  {
+    // initial R, plus the gradient of the last block state if the first chunk of a reverse pass ends a block
+    TileRegs t_init, t_inj;
+    tile_load(t_init, p.R0 ? p.R0 + (size_t)bh * mat : nullptr, true);
+    const bool inj = BLOCKS && p.Bin && ends_block(cur.t0 + cur.L);
+    tile_load(t_inj, inj ? block_matrix(p.Bin, cur.t0 + cur.L) : nullptr, inj);
+    if (p.R0) tile_accumulate(t_init, 0, false);
+    if (inj) tile_accumulate(t_inj, 0, true);
+  }
   write_rt(0);
   store_transposed(setA, 0, cur.L);
   store_rowmajor(setA, 0);
+  if (!DEEP) prefetch(setA, nxt.t0, nxt.L, nxt.ok);
   fprt::block_sync();
 
   int Lg_cached = -1;
@@ -435,7 +525,11 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const int s = it & 1;
     fprt::prof_stamp(it, 0);
     const Chunk nn = chunk_after(nxt);
-    prefetch(refill, nn.t0, nn.L, nn.ok);
+    if (DEEP) prefetch(refill, nn.t0, nn.L, nn.ok);
+    // gradient of the block state that the next chunk ends (reverse pass); an empty view otherwise
+    const bool inj = BLOCKS && p.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
+    TileRegs t_inj;
+    if (BLOCKS) tile_load(t_inj, inj ? block_matrix(p.Bin, nxt.t0 + nxt.L) : nullptr, inj);
 
     if (dbg & 4) {
       fprt::block_sync();
@@ -506,23 +600,17 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc[nq]);
     }
     store_rowmajor(ready, s ^ 1);
+    if (!DEEP) prefetch(refill, nn.t0, nn.L, nn.ok);   // refill and ready are the same set here
     fprt::sched_fence();
 
-    // state after every full block (forward walk)
+    // ---- phase 3: the state after a full block leaves (forward walk), the gradient of the next
+    // block state joins (reverse walk), and the bf16 copy for the next chunk's read-out is written.
+    // All three use this wave's part of the other stage's R buffer, in this order.
     const int t1 = cur.t0 + cur.L;
-    if (p.Bout && bs > 0 && (t1 % bs) == 0) {
-      uint16_t* dst = p.Bout + (((size_t)b * p.nblk + (t1 / bs - 1)) * p.H + h) * mat;
-#pragma unroll
-      for (int nq = 0; nq < NNW; ++nq) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dst[state_off(nq, r)] = float_to_bf16_bits(racc[nq][r]);
-      }
-    }
+    if (BLOCKS && p.Bout && ends_block(t1)) tile_store(const_cast<uint16_t*>(block_matrix(p.Bout, t1)), s ^ 1);
     fprt::prof_stamp(it, 3);
-
-    // ---- phase 3: bf16 copy of the new state for the next chunk's read-out
     if (nxt.ok) {
-      inject(nxt.t0 + nxt.L);
+      if (BLOCKS && inj) tile_accumulate(t_inj, s ^ 1, true);
       write_rt(s ^ 1);
     }
     fprt::prof_stamp(it, 4);
@@ -542,18 +630,12 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     return true;
   };
   for (int it = 0;; it += 2) {
-    if (!iteration(it, setA, setB)) break;
-    if (!iteration(it + 1, setB, setA)) break;
+    if (!iteration(it, setA, DEEP ? setB : setA)) break;
+    if (!iteration(it + 1, DEEP ? setB : setA, setA)) break;
   }
 
-  if (p.Rout) {
-    uint16_t* dst = p.Rout + (size_t)bh * mat;
-#pragma unroll
-    for (int nn = 0; nn < NNW; ++nn) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dst[state_off(nn, r)] = float_to_bf16_bits(racc[nn][r]);
-    }
-  }
+  // final R; the staging buffers are idle after the last barrier
+  if (p.Rout) tile_store(p.Rout + (size_t)bh * mat, 0);
 }
 
 }  // namespace fpk

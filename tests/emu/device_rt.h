@@ -77,6 +77,8 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 FP_DEVICE float exp2_approx(float x) { return std::exp2(x); }
 
 FP_DEVICE void sched_fence() {}
+// lanes are independent OS threads here, so lane-to-lane exchange through LDS needs a real barrier
+FP_DEVICE void wave_sync() { pthread_barrier_wait(&g_lane.wave->bar); }
 
 FP_DEVICE int dbg_flags() { return 0; }
 FP_DEVICE void prof_stamp(int, int) {}

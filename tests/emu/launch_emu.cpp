@@ -46,11 +46,14 @@ int run_grid(int nthreads, int nwg, int lds_bytes, Body body) {
 
 int fpk_launch_pass(const fpk::PassArgs& a, void* /*stream*/, const char** err) {
   const int nwg = a.B * a.H * (a.dB / fpk::BV);
+  const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   switch (a.dA) {
     case 64:
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64>(a, l); });
+      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, true>(a, l); });
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, false>(a, l); });
     case 128:
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128>(a, l); });
+      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, true>(a, l); });
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, false>(a, l); });
     case 256:
       return run_grid(fpk::NTHREADS, nwg, fpk::lds_bytes(256), [&](char* l) { fpk::retention_pass<256>(a, l); });
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
