@@ -296,7 +296,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   // Two register sets of loaded chunks, so that global loads run two chunks ahead of the math.
   // The block-state instantiation needs the registers of the second set for the block-state
   // tile in flight and keeps its loads one chunk ahead instead.
-  constexpr bool DEEP = !BLOCKS;
+  constexpr bool DEEP = true;
   struct ChunkRegs {
     u32x4 x[NXP], w[4];
     u32x2 z[4];
@@ -341,6 +341,11 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   uint32_t tile_goff[NP];                        // byte offsets inside one state matrix (< 256 KiB)
   int tile_soff[NP];                             // element offsets inside one staging stage
   auto stage_elem = [&](int e) { return (32 * nb0 + e / 32) * RT_LD + 32 * ablk + e % 32; };
+  // accumulator element (nn, r) in the staging area: one per-lane base plus constants
+  const int dl_base = tposed ? (32 * nb0 + c) * RT_LD + 32 * ablk + 4 * g
+                             : (32 * nb0 + NNW * 4 * g) * RT_LD + 32 * ablk + c;
+  auto dl_plain = [&](int nn, int r) { return dl_base + (NNW * (8 * (r >> 2) + (r & 3)) + nn) * RT_LD; };
+  auto dl_tposed = [&](int nn, int qd) { return dl_base + 32 * nn * RT_LD + 8 * qd; };
 #pragma unroll
   for (int u = 0; u < NP; ++u) {
     const int q = lane + 64 * u;
@@ -371,13 +376,13 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       if (!tposed) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float x = bf16_bits_to_float(reinterpret_cast<const u16_m*>(st)[stage_elem(acc_row(r, g) * NCOL + 32 * nn + c)]);
+          const float x = bf16_bits_to_float(reinterpret_cast<const u16_m*>(st)[dl_plain(nn, r)]);
           racc[nn][r] = add ? racc[nn][r] + x : x;
         }
       } else {
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
-          const u32x2 d = ld64(st + stage_elem((32 * nn + c) * 32 + 8 * qd + 4 * g));
+          const u32x2 d = ld64(st + dl_tposed(nn, qd));
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
             const uint32_t w = d[k >> 1];
@@ -397,14 +402,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       if (!tposed) {
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          reinterpret_cast<u16_m*>(st)[stage_elem(acc_row(r, g) * NCOL + 32 * nn + c)] = float_to_bf16_bits(racc[nn][r]);
+          reinterpret_cast<u16_m*>(st)[dl_plain(nn, r)] = float_to_bf16_bits(racc[nn][r]);
       } else {
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           u32x2 d;
           d[0] = fprt::pack_bf16x2(racc[nn][4 * qd], racc[nn][4 * qd + 1]);
           d[1] = fprt::pack_bf16x2(racc[nn][4 * qd + 2], racc[nn][4 * qd + 3]);
-          st64(st + stage_elem((32 * nn + c) * 32 + 8 * qd + 4 * g), d);
+          st64(st + dl_tposed(nn, qd), d);
         }
       }
     }
