@@ -187,7 +187,18 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 1 GiB device copy (scales the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
+    if args.copy_calibration:
+        import torch
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": src.numel()}))
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
     out = gpu_leg(args)

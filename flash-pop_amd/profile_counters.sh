@@ -1,0 +1,21 @@
+#!/bin/bash
+# Collects the rocprofv3 evidence for the pass kernel on BASELINE config 2 (run from the repo
+# root on a GPU box): kernel-trace statistics, then hardware counters in separate passes (one
+# counter group per run), then the same HBM counters on a plain copy of known size for scaling.
+# Raw output goes to gpurun_out/profile/; the figures are summarised by hand into profiles/.
+set -e
+R=$(cd "$(dirname "$0")/.." && pwd)
+O=$R/gpurun_out/profile
+mkdir -p "$O"
+cd /tmp && export TMPDIR=/tmp
+BENCH="python3 $R/bench.py --steps 5 --warmup 2 --no-cpu --no-pop"
+COPY="python3 $R/bench.py --copy-calibration"
+run() { name=$1; shift; timeout -s KILL 120 rocprofv3 "$@" --output-format csv -d "$O/$name" -o r -- $CMD > "$O/$name.log" 2>&1; }
+CMD=$BENCH run trace --kernel-trace --stats
+CMD=$BENCH run sq1 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_INSTS_LDS SQ_INSTS_SALU SQ_WAIT_INST_LDS
+CMD=$BENCH run sq2 --pmc SQ_ACTIVE_INST_VALU SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_WAIT_INST_ANY SQ_WAIT_ANY SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU_MFMA_MOPS_BF16
+CMD=$BENCH run fetch --pmc FETCH_SIZE
+CMD=$BENCH run write --pmc WRITE_SIZE
+CMD=$COPY run copy_fetch --pmc FETCH_SIZE
+CMD=$COPY run copy_write --pmc WRITE_SIZE
+echo "done: $O"
