@@ -102,12 +102,14 @@ def gpu_leg(args):
         "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "retention_pass_kernel<128>",
+            "kernel": "retention_pass_ws_kernel<128, false>",
             "achieved": round(achieved_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            # HBM bytes per launch from FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy
+            # (profiles/retention_pass_ws_kernel_128_config2.md); the same for every run of this shape
+            "traffic": 542.4e6,
             "launches_per_step": launches,
             "avg_launch_ms": round(avg_launch_ms, 4),
             "algorithmic_bytes_per_launch": (b_fwd + b_bwd) // launches,
