@@ -12,7 +12,7 @@ import numpy as np
 import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-B, T, H, DK, DV, BLOCK = 2, 150, 3, 64, 128, 64
+B, T, H, DK, DV, BLOCK = 1, 150, 2, 64, 64, 64
 DECAYS = tuple(1.0 - 2.0 ** (-5 - h) for h in range(H))
 
 
