@@ -6,10 +6,10 @@
 namespace {
 
 // dA = 64, 128: wave-specialised, 8 waves, double-buffered LDS.
-template <int DA, bool BLOCKS>
+template <int DA, bool BLOCKS, bool MULTI>
 __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::retention_pass_ws<DA, BLOCKS>(args, lds);
+  fpk::retention_pass_ws<DA, BLOCKS, MULTI>(args, lds);
 }
 
 // dA = 256: 4 symmetric waves, single-buffered LDS (two stages of 256-wide tiles do not fit).
@@ -37,7 +37,7 @@ int launch(Kernel kernel, int threads, int lds, int* armed_device, const fpk::Pa
     }
     *armed_device = dev;
   }
-  const int nwg = a.B * a.H * (a.dB / fpk::BV);
+  const int nwg = a.slots * a.H * (a.dB / fpk::BV);
   hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -60,19 +60,53 @@ extern "C" int fpk_dbg_set(int flags) {
 }
 #endif
 
-int fpk_launch_pass(const fpk::PassArgs& a, void* stream, const char** err) {
+// Compute units of the current device (cached per thread and device).
+static int compute_units() {
+  static thread_local int dev_cached = -1, cus = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev != dev_cached) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    dev_cached = dev;
+  }
+  return cus;
+}
+
+int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  static thread_local int armed[5] = {-1, -1, -1, -1, -1};
+  static thread_local int armed[7] = {-1, -1, -1, -1, -1, -1, -1};
+  fpk::PassArgs a = args;
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
+  const bool ws = a.dA == 64 || a.dA == 128;
+  // One workgroup per (batch entry, head, column tile) while that fits the chip once; beyond that
+  // the plain wave-specialised kernel lets each workgroup walk several batch entries, which keeps
+  // its load pipeline full across short sequences.
+  if (a.slots <= 0) {
+    a.slots = a.B;
+    if (ws && !blocks) {
+      const int per_slot = a.H * (a.dB / fpk::BV);
+      int fit = compute_units() / per_slot;
+      if (fit < 1) fit = 1;
+      if (fit < a.B) a.slots = fit;
+    }
+  }
+  if (a.slots > a.B) a.slots = a.B;
+  const bool multi = a.slots < a.B;
+  if (multi && (!ws || blocks)) {
+    *err = "several batch entries per workgroup need the plain wave-specialised kernel";
+    return 1;
+  }
   switch (a.dA) {
     case 64:
-      if (blocks) return launch(retention_pass_ws_kernel<64, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
-      return launch(retention_pass_ws_kernel<64, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<64, true, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
+      if (multi) return launch(retention_pass_ws_kernel<64, false, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
+      return launch(retention_pass_ws_kernel<64, false, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[2], a, s, err);
     case 128:
-      if (blocks) return launch(retention_pass_ws_kernel<128, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[2], a, s, err);
-      return launch(retention_pass_ws_kernel<128, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<128, true, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
+      if (multi) return launch(retention_pass_ws_kernel<128, false, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[4], a, s, err);
+      return launch(retention_pass_ws_kernel<128, false, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[5], a, s, err);
     case 256:
-      return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[4], a, s, err);
+      return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[6], a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }

@@ -38,6 +38,8 @@ struct PassArgs {
   int nblk;              // number of full blocks (T / block), 0 if block == 0
   int block;             // block size in tokens; chunks never straddle a multiple of it (0: none)
   int reverse;
+  int slots;             // workgroups per (head, column tile); workgroup `slot` walks the batch entries
+                         // slot, slot + slots, ... one after another.  0: the launcher chooses.
   float s_intra, s_read, s_update;
   float log2g[MAX_HEADS];
 };

@@ -45,7 +45,9 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 
 // BLOCKS: the pass writes block states (Bout) or reads their gradients (Bin).  Kept out of the
 // plain instantiation, whose state waves have no registers to spare for it.
-template <int DA, bool BLOCKS>
+// MULTI: a workgroup walks several batch entries (p.slots < p.B), so that short sequences keep
+// the load pipeline full across sequence boundaries.
+template <int DA, bool BLOCKS, bool MULTI>
 FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
   constexpr int X_LD = DA + 8;
@@ -75,8 +77,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   int wg = fprt::block_index();
   if ((nwg & 7) == 0) wg = (wg & 7) * (nwg >> 3) + (wg >> 3);   // column tiles of a stream share an XCD
   const int tile = wg % ntile;
-  const int bh = wg / ntile;
-  const int h = bh % p.H, b = bh / p.H;
+  const int h = (wg / ntile) % p.H;
+  const int slot = (wg / ntile) / p.H;   // first batch entry of this workgroup
 
   const int dbg = fprt::dbg_flags();   // always 0 outside profiling builds
   const int T = p.T, bs = p.block;
@@ -106,8 +108,28 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   auto next_pos = [&](int t0, int L) { return rev ? t0 : t0 + L; };
   auto has_more = [&](int pos) { return rev ? pos > 0 : pos < T; };
 
-  int t0, L;
-  chunk_at(rev ? T : 0, t0, L);
+  // The walk: all chunks of batch entry `slot`, then of slot + slots, ... Both roles step
+  // through the same list.
+  struct Chunk {
+    int b, t0, L;
+    bool ok, first, last;   // exists / first chunk of its sequence / last chunk of its sequence
+  };
+  auto first_chunk = [&](int b) {
+    Chunk ck = {b, 0, 0, b < p.B, true, false};
+    if (ck.ok) {
+      chunk_at(rev ? T : 0, ck.t0, ck.L);
+      ck.last = !has_more(next_pos(ck.t0, ck.L));
+    }
+    return ck;
+  };
+  auto chunk_after = [&](const Chunk& ck) {
+    if (!ck.ok) return ck;
+    if (ck.last) return MULTI ? first_chunk(ck.b + p.slots) : Chunk{ck.b, 0, 0, false, false, false};
+    Chunk n = {ck.b, 0, 0, true, false, false};
+    chunk_at(next_pos(ck.t0, ck.L), n.t0, n.L);
+    n.last = !has_more(next_pos(n.t0, n.L));
+    return n;
+  };
 
   if (!state_role) {
     // =============================== readout waves ===============================
@@ -144,8 +166,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const float wread_fwd = p.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
 
     fprt::block_sync();   // stage 0 is filled
+    Chunk ck = first_chunk(slot);
     for (int it = 0;; ++it) {
       const int s = it & 1;
+      const int L = ck.L;
       const uint16_t* xs = XS + s * CH * X_LD;
       const uint16_t* ws = WS + s * CH * X_LD;
       const uint16_t* zt = ZT + s * BV * T_LD;
@@ -162,9 +186,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       fprt::prof_stamp(it, 0);
       if (dbg & 2) {
         fprt::block_sync();
-        const int pos = next_pos(t0, L);
-        if (!has_more(pos)) break;
-        chunk_at(pos, t0, L);
+        ck = chunk_after(ck);
+        if (!ck.ok) break;
         continue;
       }
       // ---- phase 0: request X, R and the diagonal W tile
@@ -247,9 +270,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 
       fprt::block_sync();
       fprt::prof_stamp(it, 5);
-      const int pos = next_pos(t0, L);
-      if (!has_more(pos)) break;
-      chunk_at(pos, t0, L);
+      ck = chunk_after(ck);
+      if (!ck.ok) break;
     }
     return;
   }
@@ -263,12 +285,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   uint16_t* const wt = WT + sub * 32 * T_LD;
 
   const uint32_t rowA = (uint32_t)p.H * p.dA * 2, rowB = (uint32_t)p.H * p.dB * 2;   // bytes
-  const size_t streamA = ((size_t)b * T * p.H + h) * p.dA;
-  const size_t streamB = ((size_t)b * T * p.H + h) * p.dB + (size_t)tile * BV;
-  const char* const Xg = reinterpret_cast<const char*>(p.X + streamA);
-  const char* const Wg = reinterpret_cast<const char*>(p.W + streamA);
-  const char* const Zg = reinterpret_cast<const char*>(p.Z + streamB);
-  char* const Yg = reinterpret_cast<char*>(p.Y + streamB);
+  // byte offset of row t0 of sequence (b, h) in an [B,T,H,dA] tensor, resp. of this tile's columns
+  // in an [B,T,H,dB] tensor
+  auto rowsA = [&](int b, int t0) { return (((size_t)b * T + t0) * p.H + h) * p.dA * 2; };
+  auto rowsB = [&](int b, int t0) { return ((((size_t)b * T + t0) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
+  const char* const Xg = reinterpret_cast<const char*>(p.X);
+  const char* const Wg = reinterpret_cast<const char*>(p.W);
+  const char* const Zg = reinterpret_cast<const char*>(p.Z);
+  char* const Yg = reinterpret_cast<char*>(p.Y);
   const size_t mat = (size_t)p.dA * p.dB;
 
   // per-thread coordinates, bytes relative to the chunk's first row; they never change
@@ -304,12 +328,12 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   ChunkRegs setA, setB;
   // Loads are issued unconditionally so that the number of outstanding memory operations is the
   // same in every iteration; a chunk that does not exist gets zero-length views (no traffic).
-  auto prefetch = [&](ChunkRegs& cr, int ct0, int cL, bool ok) {
+  auto prefetch = [&](ChunkRegs& cr, const Chunk& ck) {
     // views that start at the chunk's first row and end with its last: later rows read as zero
-    const bool live = ok && !(dbg & 1);
-    const uint32_t lenA = live ? (uint32_t)(cL - 1) * rowA + p.dA * 2 : 0u;
-    const uint32_t lenB = live ? (uint32_t)(cL - 1) * rowB + BV * 2 : 0u;
-    const size_t baseA = (size_t)ct0 * rowA, baseB = (size_t)ct0 * rowB;
+    const bool live = ck.ok && !(dbg & 1);
+    const uint32_t lenA = live ? (uint32_t)(ck.L - 1) * rowA + p.dA * 2 : 0u;
+    const uint32_t lenB = live ? (uint32_t)(ck.L - 1) * rowB + BV * 2 : 0u;
+    const size_t baseA = live ? rowsA(ck.b, ck.t0) : 0, baseB = live ? rowsB(ck.b, ck.t0) : 0;
     const fprt::BufView xb = fprt::make_buf(Xg + baseA, lenA), wb = fprt::make_buf(Wg + baseA, lenA),
                         zb = fprt::make_buf(Zg + baseB, lenB);
 #pragma unroll
@@ -420,9 +444,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     fprt::wave_sync();   // the staging area is reused right after
   };
   // block-state matrix of the block that ends at token t1 (its gradient in a reverse pass)
-  auto block_matrix = [&](const uint16_t* base, int t1) {
+  auto block_matrix = [&](const uint16_t* base, int b, int t1) {
     return base + (((size_t)b * p.nblk + (t1 / bs - 1)) * p.H + h) * mat;
   };
+  auto state_matrix = [&](const uint16_t* base, int b) { return base + ((size_t)b * p.H + h) * mat; };
   auto ends_block = [&](int t1) { return bs > 0 && (t1 % bs) == 0; };
 
   // bf16 copy of R -> LDS stage s
@@ -489,37 +514,22 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   };
 
   // ---- prologue: chunk 0 into stage 0, chunk 1 in flight ----------------------------------
-  struct Chunk {
-    int t0, L;
-    bool ok;
-  };
-  auto chunk_after = [&](const Chunk& ck) {
-    Chunk n = {0, 0, false};
-    if (ck.ok) {
-      const int pos = next_pos(ck.t0, ck.L);
-      if (has_more(pos)) {
-        n.ok = true;
-        chunk_at(pos, n.t0, n.L);
-      }
-    }
-    return n;
-  };
-  Chunk cur = {t0, L, true}, nxt = chunk_after(cur), prev = {0, 0, false};
-  prefetch(setA, cur.t0, cur.L, true);
-  if (DEEP) prefetch(setB, nxt.t0, nxt.L, nxt.ok);
+  Chunk cur = first_chunk(slot), nxt = chunk_after(cur), prev = {0, 0, 0, false, false, false};
+  prefetch(setA, cur);
+  if (DEEP) prefetch(setB, nxt);
   {
     // initial R, plus the gradient of the last block state if the first chunk of a reverse pass ends a block
     TileRegs t_init, t_inj;
-    tile_load(t_init, p.R0 ? p.R0 + (size_t)bh * mat : nullptr, true);
+    tile_load(t_init, p.R0 ? state_matrix(p.R0, cur.b) : nullptr, true);
     const bool inj = BLOCKS && p.Bin && ends_block(cur.t0 + cur.L);
-    tile_load(t_inj, inj ? block_matrix(p.Bin, cur.t0 + cur.L) : nullptr, inj);
+    tile_load(t_inj, inj ? block_matrix(p.Bin, cur.b, cur.t0 + cur.L) : nullptr, inj);
     if (p.R0) tile_accumulate(t_init, 0, false);
     if (inj) tile_accumulate(t_inj, 0, true);
   }
   write_rt(0);
   store_transposed(setA, 0, cur.L);
   store_rowmajor(setA, 0);
-  if (!DEEP) prefetch(setA, nxt.t0, nxt.L, nxt.ok);
+  if (!DEEP) prefetch(setA, nxt);
   fprt::block_sync();
 
   int Lg_cached = -1;
@@ -530,11 +540,15 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const int s = it & 1;
     fprt::prof_stamp(it, 0);
     const Chunk nn = chunk_after(nxt);
-    if (DEEP) prefetch(refill, nn.t0, nn.L, nn.ok);
+    if (DEEP) prefetch(refill, nn);
     // gradient of the block state that the next chunk ends (reverse pass); an empty view otherwise
     const bool inj = BLOCKS && p.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
     TileRegs t_inj;
-    if (BLOCKS) tile_load(t_inj, inj ? block_matrix(p.Bin, nxt.t0 + nxt.L) : nullptr, inj);
+    if (BLOCKS) tile_load(t_inj, inj ? block_matrix(p.Bin, nxt.b, nxt.t0 + nxt.L) : nullptr, inj);
+    // initial state of the next sequence, if the next chunk starts one
+    const bool fresh = MULTI && nxt.ok && nxt.first;
+    TileRegs t_init;
+    if (MULTI) tile_load(t_init, (fresh && p.R0) ? state_matrix(p.R0, nxt.b) : nullptr, fresh);
 
     if (dbg & 4) {
       fprt::block_sync();
@@ -589,8 +603,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     {
       // rows beyond the chunk's length fall outside the view and are dropped; before the first
       // chunk the view is empty
-      const fprt::BufView yview =
-          fprt::make_buf(Yg + (size_t)prev.t0 * rowB, prev.ok ? (uint32_t)(prev.L - 1) * rowB + BV * 2 : 0u);
+      const fprt::BufView yview = fprt::make_buf(Yg + (prev.ok ? rowsB(prev.b, prev.t0) : 0),
+                                                 prev.ok ? (uint32_t)(prev.L - 1) * rowB + BV * 2 : 0u);
       fprt::buf_store128(yview, yg_off, yv[0]);
       fprt::buf_store128(yview, yg_off + 16, yv[1]);
     }
@@ -605,16 +619,26 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc[nq]);
     }
     store_rowmajor(ready, s ^ 1);
-    if (!DEEP) prefetch(refill, nn.t0, nn.L, nn.ok);   // refill and ready are the same set here
+    if (!DEEP) prefetch(refill, nn);   // refill and ready are the same set here
     fprt::sched_fence();
 
-    // ---- phase 3: the state after a full block leaves (forward walk), the gradient of the next
-    // block state joins (reverse walk), and the bf16 copy for the next chunk's read-out is written.
-    // All three use this wave's part of the other stage's R buffer, in this order.
+    // ---- phase 3: the state after a full block or at the end of a sequence leaves, the gradient
+    // of the next block state joins (reverse walk) or the next sequence's initial state takes
+    // over, and the bf16 copy for the next chunk's read-out is written.  All of them use this
+    // wave's part of the other stage's R buffer, in this order.
     const int t1 = cur.t0 + cur.L;
-    if (BLOCKS && p.Bout && ends_block(t1)) tile_store(const_cast<uint16_t*>(block_matrix(p.Bout, t1)), s ^ 1);
+    if (BLOCKS && p.Bout && ends_block(t1)) tile_store(const_cast<uint16_t*>(block_matrix(p.Bout, cur.b, t1)), s ^ 1);
+    if (cur.last && p.Rout) tile_store(const_cast<uint16_t*>(state_matrix(p.Rout, cur.b)), s ^ 1);
     fprt::prof_stamp(it, 3);
     if (nxt.ok) {
+      if (MULTI && fresh) {
+        if (p.R0) {
+          tile_accumulate(t_init, s ^ 1, false);
+        } else {
+#pragma unroll
+          for (int nq = 0; nq < NNW; ++nq) racc[nq] = f32x16{0};
+        }
+      }
       if (BLOCKS && inj) tile_accumulate(t_inj, s ^ 1, true);
       write_rt(s ^ 1);
     }
@@ -624,7 +648,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (!nxt.ok) {
       // last Y tile
       const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
-      const fprt::BufView yview = fprt::make_buf(Yg + (size_t)cur.t0 * rowB, (uint32_t)(cur.L - 1) * rowB + BV * 2);
+      const fprt::BufView yview = fprt::make_buf(Yg + rowsB(cur.b, cur.t0), (uint32_t)(cur.L - 1) * rowB + BV * 2);
       fprt::buf_store128(yview, yg_off, ld128(src));
       fprt::buf_store128(yview, yg_off + 16, ld128(src + 8));
       return false;
@@ -638,9 +662,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (!iteration(it, setA, DEEP ? setB : setA)) break;
     if (!iteration(it + 1, DEEP ? setB : setA, setA)) break;
   }
-
-  // final R; the staging buffers are idle after the last barrier
-  if (p.Rout) tile_store(p.Rout + (size_t)bh * mat, 0);
 }
 
 }  // namespace fpk

@@ -33,6 +33,8 @@ def _check_all(pairs):
     (2, 64, 1, 128, 64, 0.0),       # exactly one chunk, zero state
     (1, 70, 1, 256, 64, 0.3),       # widest contraction
     (1, 5, 3, 64, 64, 0.5),         # shorter than a chunk
+    (5, 16, 1, 128, 128, 0.5),      # several short sequences per workgroup (suffix-like), odd count
+    (4, 100, 1, 64, 128, None),     # several multi-chunk sequences per workgroup, no initial state
 ])
 def test_plain_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std):
     decays = oracle.head_decays(H)
