@@ -8,10 +8,13 @@
 //                         -> Y tile into LDS.  2 x 2 grid: `ib` = 32 chunk rows, `nb` = 32 columns.
 //                         Branch-free: every wave computes both 32 x 32 score tiles of its rows;
 //                         the tile outside the decay window is cleared after conversion.
-//   state waves   (4..7)  all global traffic (bounds-checked buffer loads two chunks ahead in
-//                         registers, Y tile stores), the transposes of W and Z into LDS, the
-//                         state update R = gamma^L R + (wkey W)^T Z in fp32 accumulators and its
-//                         bf16 copy for the read-out.
+//                         They also feed X and Z: bounds-checked buffer loads two chunks ahead in
+//                         registers, X copied and Z transposed into LDS, and they store the Y tile
+//                         of the previous chunk.
+//   state waves   (4..7)  the W traffic (loads two chunks ahead, row-major copy and the weighted
+//                         transpose into LDS), the state update R = gamma^L R + (wkey W)^T Z in
+//                         fp32 accumulators and its bf16 copy for the read-out, block states.
+// The split keeps the two roles' instruction streams about equally long.
 //
 // LDS tiles are double-buffered: while the readout waves work on chunk i from stage i & 1 the
 // state waves finish chunk i's state update and fill stage (i + 1) & 1 with chunk i + 1.  One
@@ -131,6 +134,12 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     return n;
   };
 
+  const uint32_t rowA = (uint32_t)p.H * p.dA * 2, rowB = (uint32_t)p.H * p.dB * 2;   // row pitch in bytes
+  // byte offset of row t0 of sequence (b, h) in an [B,T,H,dA] tensor, resp. of this tile's columns
+  // in an [B,T,H,dB] tensor
+  auto rowsA = [&](int b, int t0) { return (((size_t)b * T + t0) * p.H + h) * p.dA * 2; };
+  auto rowsB = [&](int b, int t0) { return ((((size_t)b * T + t0) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
+
   if (!state_role) {
     // =============================== readout waves ===============================
     const int ib = wave >> 1, nb = wave & 1;
@@ -165,11 +174,90 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const int y_off = i_row * YB_LD + 32 * nb + 4 * g;
     const float wread_fwd = p.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
 
+    // ---- feeding X, Z and draining Y: coordinates of this thread, bytes from the chunk's first row
+    const char* const Xg = reinterpret_cast<const char*>(p.X);
+    const char* const Zg = reinterpret_cast<const char*>(p.Z);
+    char* const Yg = reinterpret_cast<char*>(p.Y);
+    uint32_t xg_off[NXP];
+    int xs_off[NXP];
+#pragma unroll
+    for (int u = 0; u < NXP; ++u) {
+      const int q = tid + 256 * u, row = q / FG, col = q % FG;
+      xg_off[u] = row * rowA + col * 16;
+      xs_off[u] = row * X_LD + col * 8;
+    }
+    const int z_tg = tid >> 4, z_fq = tid & 15;      // Z unit: tokens 4 z_tg.., columns 4 z_fq..
+    uint32_t zg_off[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) zg_off[r] = (4 * z_tg + r) * rowB + z_fq * 8;
+    const int zt_off = (4 * z_fq) * T_LD + 4 * z_tg;
+    const int y_row = tid >> 2, y_col = (tid & 3) * 16;
+    const uint32_t yg_off = y_row * rowB + y_col * 2;
+
+    // Two register sets, so that the loads run two chunks ahead.  Loads and stores are issued
+    // unconditionally (zero-length views when there is nothing to do): exact wait counts.
+    struct FeedRegs {
+      u32x4 x[NXP];
+      u32x2 z[4];
+    };
+    auto feed_load = [&](FeedRegs& fr, const Chunk& c2) {
+      const bool live = c2.ok && !(dbg & 1);
+      const uint32_t lenA = live ? (uint32_t)(c2.L - 1) * rowA + p.dA * 2 : 0u;
+      const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
+      const fprt::BufView xv = fprt::make_buf(Xg + (live ? rowsA(c2.b, c2.t0) : 0), lenA);
+      const fprt::BufView zv = fprt::make_buf(Zg + (live ? rowsB(c2.b, c2.t0) : 0), lenB);
+#pragma unroll
+      for (int u = 0; u < NXP; ++u) fr.x[u] = fprt::buf_load128(xv, xg_off[u]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) fr.z[r] = fprt::buf_load64(zv, zg_off[r]);
+    };
+    auto feed_store_x = [&](const FeedRegs& fr, int s) {
+      uint16_t* xs = XS + s * CH * X_LD;
+#pragma unroll
+      for (int u = 0; u < NXP; ++u) st128(xs + xs_off[u], fr.x[u]);
+    };
+    auto feed_store_z = [&](const FeedRegs& fr, int s) {
+      uint16_t* zt = ZT + s * BV * T_LD;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int w = e >> 1;
+        u32x2 d;
+        if (e & 1) {
+          d[0] = (fr.z[0][w] >> 16) | (fr.z[1][w] & 0xffff0000u);
+          d[1] = (fr.z[2][w] >> 16) | (fr.z[3][w] & 0xffff0000u);
+        } else {
+          d[0] = (fr.z[0][w] & 0xffffu) | (fr.z[1][w] << 16);
+          d[1] = (fr.z[2][w] & 0xffffu) | (fr.z[3][w] << 16);
+        }
+        st64(zt + zt_off + e * T_LD, d);
+      }
+    };
+    // Y tile of chunk c2 from LDS stage s to global; rows beyond its length are dropped
+    auto drain_y = [&](const Chunk& c2, int s) {
+      const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
+      const u32x4 v0 = ld128(src), v1 = ld128(src + 8);
+      const fprt::BufView yv = fprt::make_buf(Yg + (c2.ok ? rowsB(c2.b, c2.t0) : 0),
+                                              c2.ok ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u);
+      fprt::buf_store128(yv, yg_off, v0);
+      fprt::buf_store128(yv, yg_off + 16, v1);
+    };
+
+    Chunk ck = first_chunk(slot), ck1 = chunk_after(ck), ckp = {0, 0, 0, false, false, false};
+    FeedRegs fa, fb;
+    feed_load(fa, ck);
+    feed_load(fb, ck1);
+    feed_store_x(fa, 0);
+    feed_store_z(fa, 0);
     fprt::block_sync();   // stage 0 is filled
-    Chunk ck = first_chunk(slot);
-    for (int it = 0;; ++it) {
+
+    // One chunk.  `refill` is the register set freed by the previous iteration (it receives chunk
+    // it + 2), `ready` holds chunk it + 1.  Returns false after the last chunk.
+    auto iteration = [&](int it, FeedRegs& refill, const FeedRegs& ready) -> bool {
       const int s = it & 1;
       const int L = ck.L;
+      const Chunk ck2 = chunk_after(ck1);
+      feed_load(refill, ck2);
+      drain_y(ckp, s ^ 1);
       const uint16_t* xs = XS + s * CH * X_LD;
       const uint16_t* ws = WS + s * CH * X_LD;
       const uint16_t* zt = ZT + s * BV * T_LD;
@@ -186,9 +274,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       fprt::prof_stamp(it, 0);
       if (dbg & 2) {
         fprt::block_sync();
-        ck = chunk_after(ck);
-        if (!ck.ok) break;
-        continue;
+        ckp = ck;
+        ck = ck1;
+        ck1 = ck2;
+        return ck.ok;
       }
       // ---- phase 0: request X, R and the diagonal W tile
       u32x4 xf[KS], rf[KS], wd[KS], wo[KS], zd[2], zo[2];
@@ -209,7 +298,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       fprt::prof_stamp(it, 1);
 
       // ---- phase 2: scores^T of the diagonal tile; the other W tile and Z arrive meanwhile (the
-      // W tile takes over the registers of the R fragments)
+      // W tile takes over the registers of the R fragments); X of chunk it + 1 goes to the other stage
 #pragma unroll
       for (int t = 0; t < KS; ++t) wo[t] = ld128(ws + wo_off + 16 * t);
 #pragma unroll
@@ -220,12 +309,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       f32x16 sd = {0};
 #pragma unroll
       for (int t = 0; t < KS; ++t) sd = fprt::mfma_32x32x16_bf16(wd[t], xf[t], sd);
+      feed_store_x(ready, s ^ 1);
       fprt::sched_fence();
       fprt::prof_stamp(it, 2);
 
       // ---- phase 3: scores^T of the other tile; the read-out is scaled and P of the diagonal
-      // tile converted in its shadow.  Accumulator element r = 8 t + e is token
-      // 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the order the Z fragments are read in.
+      // tile converted in its shadow, and Z of chunk it + 1 is transposed into the other stage.
+      // Accumulator element r = 8 t + e is token 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the
+      // order the Z fragments are read in.
       f32x16 so = {0};
 #pragma unroll
       for (int t = 0; t < KS; ++t) so = fprt::mfma_32x32x16_bf16(wo[t], xf[t], so);
@@ -240,6 +331,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
           pd[t][e] = fprt::pack_bf16x2(sd[r] * mw_d[r], sd[r + 1] * mw_d[r + 1]) & keep_d[4 * t + e];
         }
       }
+      feed_store_z(ready, s ^ 1);
       fprt::sched_fence();
       fprt::prof_stamp(it, 3);
 
@@ -270,8 +362,15 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 
       fprt::block_sync();
       fprt::prof_stamp(it, 5);
-      ck = chunk_after(ck);
-      if (!ck.ok) break;
+      ckp = ck;
+      ck = ck1;
+      ck1 = ck2;
+      if (!ck.ok) drain_y(ckp, s);   // the last Y tile
+      return ck.ok;
+    };
+    for (int it = 0;; it += 2) {
+      if (!iteration(it, fa, fb)) break;
+      if (!iteration(it + 1, fb, fa)) break;
     }
     return;
   }
@@ -284,46 +383,23 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const bool ws_writer = NAB == 4 || (sub & 1) == 0; // one wave per row block fills the row-major W tile
   uint16_t* const wt = WT + sub * 32 * T_LD;
 
-  const uint32_t rowA = (uint32_t)p.H * p.dA * 2, rowB = (uint32_t)p.H * p.dB * 2;   // bytes
-  // byte offset of row t0 of sequence (b, h) in an [B,T,H,dA] tensor, resp. of this tile's columns
-  // in an [B,T,H,dB] tensor
-  auto rowsA = [&](int b, int t0) { return (((size_t)b * T + t0) * p.H + h) * p.dA * 2; };
-  auto rowsB = [&](int b, int t0) { return ((((size_t)b * T + t0) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
-  const char* const Xg = reinterpret_cast<const char*>(p.X);
   const char* const Wg = reinterpret_cast<const char*>(p.W);
-  const char* const Zg = reinterpret_cast<const char*>(p.Z);
-  char* const Yg = reinterpret_cast<char*>(p.Y);
   const size_t mat = (size_t)p.dA * p.dB;
 
   // per-thread coordinates, bytes relative to the chunk's first row; they never change
-  uint32_t xg_off[NXP];
-  int xs_off[NXP];
-#pragma unroll
-  for (int u = 0; u < NXP; ++u) {
-    const int q = rt_id + 256 * u, row = q / FG, col = q % FG;
-    xg_off[u] = row * rowA + col * 16;
-    xs_off[u] = row * X_LD + col * 8;
-  }
   const int w_fg = lane & 3, w_tg = lane >> 2;       // W unit: tokens 4 w_tg.., features 32 ablk + 8 w_fg..
-  uint32_t wg_off[4], zg_off[4];
+  uint32_t wg_off[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) wg_off[r] = (4 * w_tg + r) * rowA + (32 * ablk + 8 * w_fg) * 2;
   const int ws_off = (4 * w_tg) * X_LD + 32 * ablk + 8 * w_fg;
   const int wt_off = (8 * w_fg) * T_LD + 4 * w_tg;
-  const int z_tg = rt_id >> 4, z_fq = rt_id & 15;    // Z unit: tokens 4 z_tg.., columns 4 z_fq..
-#pragma unroll
-  for (int r = 0; r < 4; ++r) zg_off[r] = (4 * z_tg + r) * rowB + z_fq * 8;
-  const int zt_off = (4 * z_fq) * T_LD + 4 * z_tg;
-  const int y_row = rt_id >> 2, y_col = (rt_id & 3) * 16;
-  const uint32_t yg_off = y_row * rowB + y_col * 2;
 
   // Two register sets of loaded chunks, so that global loads run two chunks ahead of the math.
   // The block-state instantiation needs the registers of the second set for the block-state
   // tile in flight and keeps its loads one chunk ahead instead.
   constexpr bool DEEP = true;
   struct ChunkRegs {
-    u32x4 x[NXP], w[4];
-    u32x2 z[4];
+    u32x4 w[4];
   };
   ChunkRegs setA, setB;
   // Loads are issued unconditionally so that the number of outstanding memory operations is the
@@ -332,16 +408,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // views that start at the chunk's first row and end with its last: later rows read as zero
     const bool live = ck.ok && !(dbg & 1);
     const uint32_t lenA = live ? (uint32_t)(ck.L - 1) * rowA + p.dA * 2 : 0u;
-    const uint32_t lenB = live ? (uint32_t)(ck.L - 1) * rowB + BV * 2 : 0u;
-    const size_t baseA = live ? rowsA(ck.b, ck.t0) : 0, baseB = live ? rowsB(ck.b, ck.t0) : 0;
-    const fprt::BufView xb = fprt::make_buf(Xg + baseA, lenA), wb = fprt::make_buf(Wg + baseA, lenA),
-                        zb = fprt::make_buf(Zg + baseB, lenB);
-#pragma unroll
-    for (int u = 0; u < NXP; ++u) cr.x[u] = fprt::buf_load128(xb, xg_off[u]);
+    const fprt::BufView wb = fprt::make_buf(Wg + (live ? rowsA(ck.b, ck.t0) : 0), lenA);
 #pragma unroll
     for (int r = 0; r < 4; ++r) cr.w[r] = fprt::buf_load128(wb, wg_off[r]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) cr.z[r] = fprt::buf_load64(zb, zg_off[r]);
   };
 
   // state tiles: racc[nn] is R[32 ablk + acc_row][32 (nb0 + nn) + c]
@@ -465,11 +534,11 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     }
   };
 
-  // A loaded chunk of length cL goes to LDS stage s: the weighted W^T slab and Z^T are formed in
-  // registers and written at once (short live ranges), the row-major X and W tiles are copies.
+  // A loaded W chunk of length cL goes to LDS: the weighted W^T slab is formed in registers and
+  // written at once (short live ranges), the row-major W tile of stage s is a copy.
   int Lk_cached = -1;
   float wkey[4];
-  auto store_transposed = [&](const ChunkRegs& cr, int s, int cL) {
+  auto store_transposed = [&](const ChunkRegs& cr, int cL) {
     if (cL != Lk_cached) {
       Lk_cached = cL;
 #pragma unroll
@@ -480,7 +549,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         wkey[r] = p.s_update * fprt::exp2_approx((float)e * lg);
       }
     }
-    uint16_t* zt = ZT + s * BV * T_LD;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       u32x2 d;
@@ -488,25 +556,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       d[1] = fprt::pack_bf16x2(bf16_elem(cr.w[2], e) * wkey[2], bf16_elem(cr.w[3], e) * wkey[3]);
       st64(wt + wt_off + e * T_LD, d);
     }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int w = e >> 1;
-      u32x2 d;
-      if (e & 1) {
-        d[0] = (cr.z[0][w] >> 16) | (cr.z[1][w] & 0xffff0000u);
-        d[1] = (cr.z[2][w] >> 16) | (cr.z[3][w] & 0xffff0000u);
-      } else {
-        d[0] = (cr.z[0][w] & 0xffffu) | (cr.z[1][w] << 16);
-        d[1] = (cr.z[2][w] & 0xffffu) | (cr.z[3][w] << 16);
-      }
-      st64(zt + zt_off + e * T_LD, d);
-    }
   };
   auto store_rowmajor = [&](const ChunkRegs& cr, int s) {
-    uint16_t* xs = XS + s * CH * X_LD;
     uint16_t* ws = WS + s * CH * X_LD;
-#pragma unroll
-    for (int u = 0; u < NXP; ++u) st128(xs + xs_off[u], cr.x[u]);
     if (ws_writer) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) st128(ws + ws_off + r * X_LD, cr.w[r]);
@@ -514,7 +566,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   };
 
   // ---- prologue: chunk 0 into stage 0, chunk 1 in flight ----------------------------------
-  Chunk cur = first_chunk(slot), nxt = chunk_after(cur), prev = {0, 0, 0, false, false, false};
+  Chunk cur = first_chunk(slot), nxt = chunk_after(cur);
   prefetch(setA, cur);
   if (DEEP) prefetch(setB, nxt);
   {
@@ -527,7 +579,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (inj) tile_accumulate(t_inj, 0, true);
   }
   write_rt(0);
-  store_transposed(setA, 0, cur.L);
+  store_transposed(setA, cur.L);
   store_rowmajor(setA, 0);
   if (!DEEP) prefetch(setA, nxt);
   fprt::block_sync();
@@ -553,30 +605,24 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (dbg & 4) {
       fprt::block_sync();
       if (!nxt.ok) return false;
-      prev = cur;
       cur = nxt;
       nxt = nn;
       return true;
     }
     // ---- phase 0: request the operands of the state update (this wave's whole W^T slab, the
-    // first half of Z^T) and the finished Y tile; decay R while they arrive
+    // first half of Z^T); decay R while they arrive
     if (cur.L != Lg_cached) {
       Lg_cached = cur.L;
       gL = fprt::exp2_approx((float)cur.L * lg);
     }
     const uint16_t* zt = ZT + s * BV * T_LD;
-    u32x4 wf[4], zlo[NNW][2], zhi[NNW][2], yv[2];
+    u32x4 wf[4], zlo[NNW][2], zhi[NNW][2];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) wf[kt] = ld_token_frag(wt + c * T_LD + 16 * kt + 4 * g);
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int nq = 0; nq < NNW; ++nq) zlo[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * kt + 4 * g);
-    }
-    {
-      const uint16_t* src = YB + (s ^ 1) * CH * YB_LD + y_row * YB_LD + y_col;
-      yv[0] = ld128(src);
-      yv[1] = ld128(src + 8);
     }
 #pragma unroll
     for (int nq = 0; nq < NNW; ++nq) {
@@ -587,8 +633,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     fprt::prof_stamp(it, 1);
 
     // ---- phase 1: first half of R = gamma^L R + (wkey W)^T Z; in its shadow the rest of Z^T is
-    // requested, the previous Y tile leaves, and chunk it + 1 (zeros if there is none) is
-    // transposed into the other stage.  The W^T slab is overwritten only after all of it was read.
+    // requested and the W of chunk it + 1 (zeros if there is none) is transposed.  The W^T slab is overwritten only after all of it was read.
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
@@ -600,15 +645,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       for (int nq = 0; nq < NNW; ++nq)
         zhi[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * (2 + kt) + 4 * g);
     }
-    {
-      // rows beyond the chunk's length fall outside the view and are dropped; before the first
-      // chunk the view is empty
-      const fprt::BufView yview = fprt::make_buf(Yg + (prev.ok ? rowsB(prev.b, prev.t0) : 0),
-                                                 prev.ok ? (uint32_t)(prev.L - 1) * rowB + BV * 2 : 0u);
-      fprt::buf_store128(yview, yg_off, yv[0]);
-      fprt::buf_store128(yview, yg_off + 16, yv[1]);
-    }
-    store_transposed(ready, s ^ 1, nxt.L);
+    store_transposed(ready, nxt.L);
     fprt::sched_fence();
     fprt::prof_stamp(it, 2);
 
@@ -645,15 +682,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     fprt::prof_stamp(it, 4);
     fprt::block_sync();
     fprt::prof_stamp(it, 5);
-    if (!nxt.ok) {
-      // last Y tile
-      const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
-      const fprt::BufView yview = fprt::make_buf(Yg + rowsB(cur.b, cur.t0), (uint32_t)(cur.L - 1) * rowB + BV * 2);
-      fprt::buf_store128(yview, yg_off, ld128(src));
-      fprt::buf_store128(yview, yg_off + 16, ld128(src + 8));
-      return false;
-    }
-    prev = cur;
+    if (!nxt.ok) return false;
     cur = nxt;
     nxt = nn;
     return true;

@@ -101,5 +101,8 @@ FP_DEVICE u32x2 buf_load64(BufView b, uint32_t off) {
 FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) {
   if ((uint64_t)off + 16 <= b.nbytes) std::memcpy(const_cast<char*>(b.base) + off, &v, 16);
 }
+FP_DEVICE void buf_store64(BufView b, uint32_t off, u32x2 v) {
+  if ((uint64_t)off + 8 <= b.nbytes) std::memcpy(const_cast<char*>(b.base) + off, &v, 8);
+}
 
 }  // namespace fprt
