@@ -142,6 +142,80 @@ int backward(const Shape& s, const void* q, const void* k, const void* v, const 
   return run(a, stream, "dv");
 }
 
+// Suffix tensors of one fused POP call, in the roles q, k, v / d_o (inputs) and o / dq, dk, dv (outputs)
+struct Suffixes {
+  const void *q, *k, *v;
+  int len;
+};
+
+int check_fused(const Shape& s, int block, int sfx_len) {
+  if (block < 1) return fail(FP_ERR_BAD_SHAPE, "block_size must be >= 1 (got %d)", block);
+  if (s.T % block != 0)
+    return fail(FP_ERR_BAD_SHAPE, "the fused POP op needs T to be a multiple of block_size (got T=%d, block_size=%d)", s.T, block);
+  if (sfx_len < 1 || sfx_len > fpk::CH)
+    return fail(FP_ERR_BAD_SHAPE, "suffix length must be in 1..%d (got %d)", fpk::CH, sfx_len);
+  if (s.dk > 128 || s.dv > 128)
+    return fail(FP_ERR_UNSUPPORTED_DIM, "the fused POP op supports dk and dv of 64 or 128 (got dk=%d, dv=%d)", s.dk, s.dv);
+  return FP_OK;
+}
+
+void suffix_walk(fpk::PassArgs& a, const Shape& s, int block, int sfx_len, const void* x, const void* w, const void* z,
+                 void* y) {
+  a.block = block;
+  a.nblk = s.T / block;
+  a.Ls = sfx_len;
+  a.Xs = in(x); a.Ws = in(w); a.Zs = in(z); a.Ys = out(y);
+}
+
+int fused_forward(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const Suffixes& x,
+                  const double* decays, void* o, void* o_sfx, void* s_out, int block, void* stream) {
+  fpk::PassArgs a;
+  fill_common(a, s, decays);
+  const float sc = 1.0f / std::sqrt((float)s.dk);
+  a.X = in(q); a.W = in(k); a.Z = in(v); a.Y = out(o);
+  a.R0 = in(s0); a.Rout = out(s_out);
+  plain_state(a, s);
+  suffix_walk(a, s, block, x.len, x.q, x.k, x.v, o_sfx);
+  a.reverse = 0;
+  a.s_intra = sc; a.s_read = 1.f; a.s_update = sc;
+  return run(a, stream, "fused forward");
+}
+
+int fused_backward(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const Suffixes& x,
+                   const double* decays, const void* d_o, const void* d_o_sfx, const void* d_s_out, void* dq, void* dk_,
+                   void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx, void* d_s0, int block, void* stream) {
+  const float sc = 1.0f / std::sqrt((float)s.dk);
+  fpk::PassArgs a;
+  int rc;
+
+  fill_common(a, s, decays);   // dq
+  a.X = in(d_o); a.W = in(v); a.Z = in(k); a.Y = out(dq);
+  a.R0 = in(s0);
+  transposed_state(a, s);
+  suffix_walk(a, s, block, x.len, d_o_sfx, x.v, x.k, dq_sfx);
+  a.reverse = 0;
+  a.s_intra = sc; a.s_read = 1.f; a.s_update = sc;
+  if ((rc = run(a, stream, "fused dq")) != FP_OK) return rc;
+
+  fill_common(a, s, decays);   // dk
+  a.X = in(v); a.W = in(d_o); a.Z = in(q); a.Y = out(dk_);
+  a.R0 = in(d_s_out);
+  transposed_state(a, s);
+  suffix_walk(a, s, block, x.len, x.v, d_o_sfx, x.q, dk_sfx);
+  a.reverse = 1;
+  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
+  if ((rc = run(a, stream, "fused dk")) != FP_OK) return rc;
+
+  fill_common(a, s, decays);   // dv (+ d_s0)
+  a.X = in(k); a.W = in(q); a.Z = in(d_o); a.Y = out(dv_);
+  a.R0 = in(d_s_out); a.Rout = out(d_s0);
+  plain_state(a, s);
+  suffix_walk(a, s, block, x.len, x.k, x.q, d_o_sfx, dv_sfx);
+  a.reverse = 1;
+  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
+  return run(a, stream, "fused dv");
+}
+
 }  // namespace
 
 extern "C" {
@@ -188,8 +262,34 @@ int fp_pop_retention_bwd(const void* q, const void* k, const void* v, const void
   return backward(s, q, k, v, s0, head_decays, d_o, nullptr, d_blocks, block_size, dq, dk_, dv_, d_s0, stream);
 }
 
+int fp_pop_fused_fwd(const void* q, const void* k, const void* v, const void* s0, const void* q_sfx, const void* k_sfx,
+                     const void* v_sfx, const double* head_decays, void* o, void* o_sfx, void* s_out, int B, int T,
+                     int H, int dk, int dv, int block_size, int sfx_len, void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_fused(s, block_size, sfx_len)) return rc;
+  if (!q || !k || !v || !o || !q_sfx || !k_sfx || !v_sfx || !o_sfx)
+    return fail(FP_ERR_NULL_POINTER, "q, k, v, o and their suffix counterparts must not be NULL");
+  return fused_forward(s, q, k, v, s0, Suffixes{q_sfx, k_sfx, v_sfx, sfx_len}, head_decays, o, o_sfx, s_out, block_size,
+                       stream);
+}
+
+int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0, const void* q_sfx, const void* k_sfx,
+                     const void* v_sfx, const double* head_decays, const void* d_o, const void* d_o_sfx,
+                     const void* d_s_out, void* dq, void* dk_, void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx,
+                     void* d_s0, int B, int T, int H, int dk, int dv, int block_size, int sfx_len, void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_fused(s, block_size, sfx_len)) return rc;
+  if (!q || !k || !v || !q_sfx || !k_sfx || !v_sfx || !d_o || !d_o_sfx || !dq || !dk_ || !dv_ || !dq_sfx || !dk_sfx ||
+      !dv_sfx)
+    return fail(FP_ERR_NULL_POINTER, "inputs, d_o, d_o_sfx and the six gradient outputs must not be NULL");
+  return fused_backward(s, q, k, v, s0, Suffixes{q_sfx, k_sfx, v_sfx, sfx_len}, head_decays, d_o, d_o_sfx, d_s_out, dq,
+                        dk_, dv_, dq_sfx, dk_sfx, dv_sfx, d_s0, block_size, stream);
+}
+
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1000; }
+int fp_version(void) { return 1001; }
 
 }  // extern "C"

@@ -6,10 +6,10 @@
 namespace {
 
 // dA = 64, 128: wave-specialised, 8 waves, double-buffered LDS.
-template <int DA, bool BLOCKS, bool MULTI>
+template <int DA, int MODE>
 __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::retention_pass_ws<DA, BLOCKS, MULTI>(args, lds);
+  fpk::retention_pass_ws<DA, MODE>(args, lds);
 }
 
 // dA = 256: 4 symmetric waves, single-buffered LDS (two stages of 256-wide tiles do not fit).
@@ -74,16 +74,25 @@ static int compute_units() {
 
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  static thread_local int armed[7] = {-1, -1, -1, -1, -1, -1, -1};
+  static thread_local int armed[9] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
   fpk::PassArgs a = args;
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool ws = a.dA == 64 || a.dA == 128;
+  const bool suffix = a.Ls > 0;
+  if (suffix) {
+    // what the suffix walk assumes; the C-ABI layer reports these to the caller in its own words
+    if (!ws || blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > fpk::CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys) {
+      *err = "suffix walk: needs dA of 64 or 128, T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
+      return 1;
+    }
+    a.slots = a.B;
+  }
   // One workgroup per (batch entry, head, column tile) while that fits the chip once; beyond that
   // the plain wave-specialised kernel lets each workgroup walk several batch entries, which keeps
   // its load pipeline full across short sequences.
   if (a.slots <= 0) {
     a.slots = a.B;
-    if (ws && !blocks) {
+    if (ws && !blocks && !suffix) {
       const int per_slot = a.H * (a.dB / fpk::BV);
       int fit = compute_units() / per_slot;
       if (fit < 1) fit = 1;
@@ -92,19 +101,21 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   }
   if (a.slots > a.B) a.slots = a.B;
   const bool multi = a.slots < a.B;
-  if (multi && (!ws || blocks)) {
+  if (multi && (!ws || blocks || suffix)) {
     *err = "several batch entries per workgroup need the plain wave-specialised kernel";
     return 1;
   }
   switch (a.dA) {
     case 64:
-      if (blocks) return launch(retention_pass_ws_kernel<64, true, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
-      if (multi) return launch(retention_pass_ws_kernel<64, false, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
-      return launch(retention_pass_ws_kernel<64, false, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[2], a, s, err);
+      if (suffix) return launch(retention_pass_ws_kernel<64, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[7], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<64, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
+      if (multi) return launch(retention_pass_ws_kernel<64, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
+      return launch(retention_pass_ws_kernel<64, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[2], a, s, err);
     case 128:
-      if (blocks) return launch(retention_pass_ws_kernel<128, true, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
-      if (multi) return launch(retention_pass_ws_kernel<128, false, true>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[4], a, s, err);
-      return launch(retention_pass_ws_kernel<128, false, false>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[5], a, s, err);
+      if (suffix) return launch(retention_pass_ws_kernel<128, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[8], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
+      if (multi) return launch(retention_pass_ws_kernel<128, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[4], a, s, err);
+      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[5], a, s, err);
     case 256:
       return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[6], a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;

@@ -33,11 +33,18 @@ struct PassArgs {
   uint16_t* Rout;        // final R per (b, h), nullable
   uint16_t* Bout;        // R after every full block, [B, nblk, H, dk*dv], nullable (forward only)
   const uint16_t* Bin;   // added to R before the chunk that ends each full block, nullable (reverse only)
+  // Suffix tensors, [B, nblk + 1, Ls, H, d] in the roles of X, W, Z, Y (all four or none; Ls > 0
+  // selects the suffix walk, which needs T == nblk * block).
+  const uint16_t* Xs;
+  const uint16_t* Ws;
+  const uint16_t* Zs;
+  uint16_t* Ys;
   long long rs_a, rs_n;  // element strides of R[a][n] inside one dk*dv state matrix
   int B, T, H, dA, dB;
   int nblk;              // number of full blocks (T / block), 0 if block == 0
   int block;             // block size in tokens; chunks never straddle a multiple of it (0: none)
   int reverse;
+  int Ls;                // tokens per suffix, 1..CH; 0: no suffixes
   int slots;             // workgroups per (head, column tile); workgroup `slot` walks the batch entries
                          // slot, slot + slots, ... one after another.  0: the launcher chooses.
   float s_intra, s_read, s_update;

@@ -46,13 +46,22 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
   return u32x4{lo[0], lo[1], hi[0], hi[1]};
 }
 
-// BLOCKS: the pass writes block states (Bout) or reads their gradients (Bin).  Kept out of the
-// plain instantiation, whose state waves have no registers to spare for it.
-// MULTI: a workgroup walks several batch entries (p.slots < p.B), so that short sequences keep
-// the load pipeline full across sequence boundaries.
-template <int DA, bool BLOCKS, bool MULTI>
+// Variants of the walk, one instantiation each so that the plain one stays lean:
+// WALK_BLOCKS  the pass writes block states (Bout) or reads their gradients (Bin);
+// WALK_MULTI   a workgroup walks several batch entries (p.slots < p.B), so that short sequences
+//              keep the load pipeline full across sequence boundaries;
+// WALK_SUFFIX  a suffix of p.Ls tokens hangs off every block boundary (positions 0, block, ...,
+//              T; T is a multiple of the block size).  It is one more item of the walk, placed at
+//              its boundary, with its own tensors: it reads the state at the boundary without
+//              advancing it.  Walking forward its keys get weight 0 and R is not decayed; walking
+//              backward its read-out weight is 0 and what it adds to R (the gradient of the state
+//              it read) is not decayed either.
+enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3 };
+
+template <int DA, int MODE>
 FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
+  constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI, SFX = MODE == WALK_SUFFIX;
   constexpr int X_LD = DA + 8;
   constexpr int T_LD = CH + 4;      // row length of the transposed tiles (tokens)
   constexpr int RT_LD = DA + 8;
@@ -115,30 +124,64 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   // through the same list.
   struct Chunk {
     int b, t0, L;
-    bool ok, first, last;   // exists / first chunk of its sequence / last chunk of its sequence
+    bool ok, first, last;   // exists / first item of its sequence / last item of its sequence
+    bool sfx;               // a suffix (t0 is its block boundary) rather than a context chunk
+    int n;                  // WALK_SUFFIX only: index of the suffix, or of the context chunk's block
   };
+  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0};
   auto first_chunk = [&](int b) {
-    Chunk ck = {b, 0, 0, b < p.B, true, false};
+    Chunk ck = {b, 0, 0, b < p.B, true, false, false, 0};
     if (ck.ok) {
-      chunk_at(rev ? T : 0, ck.t0, ck.L);
-      ck.last = !has_more(next_pos(ck.t0, ck.L));
+      if (SFX) {   // the suffix at the first boundary met: position 0, or T walking backward
+        ck.sfx = true;
+        ck.n = rev ? p.nblk : 0;
+        ck.t0 = rev ? T : 0;
+        ck.L = p.Ls;
+      } else {
+        chunk_at(rev ? T : 0, ck.t0, ck.L);
+        ck.last = !has_more(next_pos(ck.t0, ck.L));
+      }
     }
     return ck;
   };
   auto chunk_after = [&](const Chunk& ck) {
     if (!ck.ok) return ck;
-    if (ck.last) return MULTI ? first_chunk(ck.b + p.slots) : Chunk{ck.b, 0, 0, false, false, false};
-    Chunk n = {ck.b, 0, 0, true, false, false};
+    if (ck.last) return MULTI ? first_chunk(ck.b + p.slots) : no_chunk;
+    Chunk n = {ck.b, 0, 0, true, false, false, false, 0};
+    if (SFX) {
+      // Block m spans [m bs, (m + 1) bs).  After a suffix comes the nearest context chunk of the
+      // block that follows it in walking order; after the context chunk that reaches the far
+      // boundary of its block comes that boundary's suffix.
+      if (!rev) {
+        const int m = ck.n, pos = ck.sfx ? ck.t0 : ck.t0 + ck.L, lim = (m + 1) * bs;
+        if (!ck.sfx && pos == lim) {
+          n.sfx = true; n.n = m + 1; n.t0 = pos; n.L = p.Ls; n.last = pos == T;
+        } else {
+          n.n = m; n.t0 = pos; n.L = (pos + CH < lim ? pos + CH : lim) - pos;
+        }
+      } else {
+        const int m = ck.sfx ? ck.n - 1 : ck.n, pos = ck.t0, lo = m * bs;
+        if (!ck.sfx && pos == lo) {
+          n.sfx = true; n.n = m; n.t0 = pos; n.L = p.Ls; n.last = pos == 0;
+        } else {
+          n.n = m; n.t0 = pos - CH > lo ? pos - CH : lo; n.L = pos - n.t0;
+        }
+      }
+      return n;
+    }
     chunk_at(next_pos(ck.t0, ck.L), n.t0, n.L);
     n.last = !has_more(next_pos(n.t0, n.L));
     return n;
   };
 
   const uint32_t rowA = (uint32_t)p.H * p.dA * 2, rowB = (uint32_t)p.H * p.dB * 2;   // row pitch in bytes
-  // byte offset of row t0 of sequence (b, h) in an [B,T,H,dA] tensor, resp. of this tile's columns
-  // in an [B,T,H,dB] tensor
-  auto rowsA = [&](int b, int t0) { return (((size_t)b * T + t0) * p.H + h) * p.dA * 2; };
-  auto rowsB = [&](int b, int t0) { return ((((size_t)b * T + t0) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
+  // byte offset of the item's first row for head h in an [B,T,H,dA] tensor (suffixes:
+  // [B, nblk + 1, Ls, H, dA]), resp. of this tile's columns in the dB-wide tensors
+  auto first_row = [&](const Chunk& ck) {
+    return (SFX && ck.sfx) ? ((size_t)ck.b * (p.nblk + 1) + ck.n) * p.Ls : (size_t)ck.b * T + ck.t0;
+  };
+  auto rowsA = [&](const Chunk& ck) { return (first_row(ck) * p.H + h) * p.dA * 2; };
+  auto rowsB = [&](const Chunk& ck) { return ((first_row(ck) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
 
   if (!state_role) {
     // =============================== readout waves ===============================
@@ -178,6 +221,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const char* const Xg = reinterpret_cast<const char*>(p.X);
     const char* const Zg = reinterpret_cast<const char*>(p.Z);
     char* const Yg = reinterpret_cast<char*>(p.Y);
+    const char* const Xsg = reinterpret_cast<const char*>(p.Xs);
+    const char* const Zsg = reinterpret_cast<const char*>(p.Zs);
+    char* const Ysg = reinterpret_cast<char*>(p.Ys);
     uint32_t xg_off[NXP];
     int xs_off[NXP];
 #pragma unroll
@@ -204,8 +250,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       const bool live = c2.ok && !(dbg & 1);
       const uint32_t lenA = live ? (uint32_t)(c2.L - 1) * rowA + p.dA * 2 : 0u;
       const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
-      const fprt::BufView xv = fprt::make_buf(Xg + (live ? rowsA(c2.b, c2.t0) : 0), lenA);
-      const fprt::BufView zv = fprt::make_buf(Zg + (live ? rowsB(c2.b, c2.t0) : 0), lenB);
+      const bool sf = SFX && c2.sfx;
+      const fprt::BufView xv = fprt::make_buf((sf ? Xsg : Xg) + (live ? rowsA(c2) : 0), lenA);
+      const fprt::BufView zv = fprt::make_buf((sf ? Zsg : Zg) + (live ? rowsB(c2) : 0), lenB);
 #pragma unroll
       for (int u = 0; u < NXP; ++u) fr.x[u] = fprt::buf_load128(xv, xg_off[u]);
 #pragma unroll
@@ -236,13 +283,13 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     auto drain_y = [&](const Chunk& c2, int s) {
       const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
       const u32x4 v0 = ld128(src), v1 = ld128(src + 8);
-      const fprt::BufView yv = fprt::make_buf(Yg + (c2.ok ? rowsB(c2.b, c2.t0) : 0),
+      const fprt::BufView yv = fprt::make_buf(((SFX && c2.sfx) ? Ysg : Yg) + (c2.ok ? rowsB(c2) : 0),
                                               c2.ok ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u);
       fprt::buf_store128(yv, yg_off, v0);
       fprt::buf_store128(yv, yg_off + 16, v1);
     };
 
-    Chunk ck = first_chunk(slot), ck1 = chunk_after(ck), ckp = {0, 0, 0, false, false, false};
+    Chunk ck = first_chunk(slot), ck1 = chunk_after(ck), ckp = no_chunk;
     FeedRegs fa, fb;
     feed_load(fa, ck);
     feed_load(fb, ck1);
@@ -269,6 +316,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         int e = L - 1 - i_row;
         if (e < 0) e = 0;
         wread = p.s_read * fprt::exp2_approx((float)e * lg);
+        if (SFX && ck.sfx) wread = 0.f;   // nothing downstream of a suffix reaches back into it
       }
 
       fprt::prof_stamp(it, 0);
@@ -384,6 +432,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   uint16_t* const wt = WT + sub * 32 * T_LD;
 
   const char* const Wg = reinterpret_cast<const char*>(p.W);
+  const char* const Wsg = reinterpret_cast<const char*>(p.Ws);
   const size_t mat = (size_t)p.dA * p.dB;
 
   // per-thread coordinates, bytes relative to the chunk's first row; they never change
@@ -408,7 +457,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // views that start at the chunk's first row and end with its last: later rows read as zero
     const bool live = ck.ok && !(dbg & 1);
     const uint32_t lenA = live ? (uint32_t)(ck.L - 1) * rowA + p.dA * 2 : 0u;
-    const fprt::BufView wb = fprt::make_buf(Wg + (live ? rowsA(ck.b, ck.t0) : 0), lenA);
+    const fprt::BufView wb = fprt::make_buf(((SFX && ck.sfx) ? Wsg : Wg) + (live ? rowsA(ck) : 0), lenA);
 #pragma unroll
     for (int r = 0; r < 4; ++r) cr.w[r] = fprt::buf_load128(wb, wg_off[r]);
   };
@@ -534,19 +583,21 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     }
   };
 
-  // A loaded W chunk of length cL goes to LDS: the weighted W^T slab is formed in registers and
-  // written at once (short live ranges), the row-major W tile of stage s is a copy.
+  // A loaded W chunk goes to LDS: the weighted W^T slab is formed in registers and written at
+  // once (short live ranges), the row-major W tile of stage s is a copy.
   int Lk_cached = -1;
   float wkey[4];
-  auto store_transposed = [&](const ChunkRegs& cr, int cL) {
-    if (cL != Lk_cached) {
-      Lk_cached = cL;
+  auto store_transposed = [&](const ChunkRegs& cr, const Chunk& ck) {
+    const bool sf = SFX && ck.sfx;
+    const int key = ck.L + (sf ? 256 : 0);
+    if (key != Lk_cached) {
+      Lk_cached = key;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int j = 4 * w_tg + r;
-        int e = rev ? (j + 1) : (cL - 1 - j);
+        int e = rev ? (j + 1) : (ck.L - 1 - j);
         if (e < 0) e = 0;
-        wkey[r] = p.s_update * fprt::exp2_approx((float)e * lg);
+        wkey[r] = (sf && !rev) ? 0.f : p.s_update * fprt::exp2_approx((float)e * lg);
       }
     }
 #pragma unroll
@@ -579,7 +630,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (inj) tile_accumulate(t_inj, 0, true);
   }
   write_rt(0);
-  store_transposed(setA, cur.L);
+  store_transposed(setA, cur);
   store_rowmajor(setA, 0);
   if (!DEEP) prefetch(setA, nxt);
   fprt::block_sync();
@@ -611,9 +662,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     }
     // ---- phase 0: request the operands of the state update (this wave's whole W^T slab, the
     // first half of Z^T); decay R while they arrive
-    if (cur.L != Lg_cached) {
-      Lg_cached = cur.L;
-      gL = fprt::exp2_approx((float)cur.L * lg);
+    const int gkey = (SFX && cur.sfx) ? 0 : cur.L;   // a suffix does not advance the state
+    if (gkey != Lg_cached) {
+      Lg_cached = gkey;
+      gL = fprt::exp2_approx((float)gkey * lg);
     }
     const uint16_t* zt = ZT + s * BV * T_LD;
     u32x4 wf[4], zlo[NNW][2], zhi[NNW][2];
@@ -645,7 +697,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       for (int nq = 0; nq < NNW; ++nq)
         zhi[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * (2 + kt) + 4 * g);
     }
-    store_transposed(ready, nxt.L);
+    store_transposed(ready, nxt);
     fprt::sched_fence();
     fprt::prof_stamp(it, 2);
 

@@ -79,3 +79,52 @@ def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size,
                                           block_size, _stream())
     _lib.check(lib, rc)
     return dq, dk_, dv_, d_s0
+
+
+def prepare_suffixes(q_sfx, k_sfx, v_sfx, shape, block_size):
+    """Checks of the suffix batch as POPDecoderLayer._suffixes_forward makes them
+    (flash_pop/pop_retnet.py:154-159): one suffix per block boundary, N + 1 per sequence."""
+    B, T, H, dk, dv = shape
+    if T % block_size != 0:
+        raise ValueError(f"the fused POP op needs T ({T}) to be a multiple of block_size ({block_size})")
+    n = B * (T // block_size + 1)
+    if q_sfx.dim() != 4 or k_sfx.shape != q_sfx.shape or v_sfx.dim() != 4 or v_sfx.shape[:3] != q_sfx.shape[:3]:
+        raise ValueError("expected q_sfx, k_sfx [B*(N+1),Ls,H,dk] and v_sfx [B*(N+1),Ls,H,dv]")
+    if q_sfx.shape[0] != n or q_sfx.shape[2] != H or q_sfx.shape[3] != dk or v_sfx.shape[3] != dv:
+        raise ValueError(f"got suffix tensors {tuple(q_sfx.shape)}, {tuple(v_sfx.shape)} for {n} suffixes of "
+                         f"{H} heads with dk={dk}, dv={dv}: make sure there is one additional suffix block")
+    for name, t in (("q_sfx", q_sfx), ("k_sfx", k_sfx), ("v_sfx", v_sfx)):
+        assert t.dtype == torch.bfloat16, f"{name}: only bfloat16 is supported, got {t.dtype}"
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}: flash_pop_amd runs on the GPU only")
+    return q_sfx.contiguous(), k_sfx.contiguous(), v_sfx.contiguous()
+
+
+def pop_fused_fwd(q, k, v, s, sfx, decays, block_size, shape):
+    lib = _lib.load()
+    B, T, H, dk, dv = shape
+    o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
+    o_sfx = torch.empty_like(sfx[2])
+    s_out = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.fp_pop_fused_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _ptr(sfx[0]), _ptr(sfx[1]), _ptr(sfx[2]),
+                                  _lib.decays_array(decays), _ptr(o), _ptr(o_sfx), _ptr(s_out), B, T, H, dk, dv,
+                                  block_size, sfx[0].shape[1], _stream())
+    _lib.check(lib, rc)
+    return o, o_sfx, s_out
+
+
+def pop_fused_bwd(q, k, v, s, sfx, decays, block_size, shape, d_o, d_o_sfx, d_s_out, want_ds0):
+    lib = _lib.load()
+    B, T, H, dk, dv = shape
+    d_o, d_o_sfx = d_o.contiguous(), d_o_sfx.contiguous()
+    d_s_out = None if d_s_out is None else d_s_out.contiguous()
+    outs = [torch.empty_like(t) for t in (q, k, v, *sfx)]
+    d_s0 = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device) if want_ds0 else None
+    with torch.cuda.device(q.device):
+        rc = lib.fp_pop_fused_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _ptr(sfx[0]), _ptr(sfx[1]), _ptr(sfx[2]),
+                                  _lib.decays_array(decays), _ptr(d_o), _ptr(d_o_sfx), _ptr(d_s_out),
+                                  *[_ptr(t) for t in outs], _ptr(d_s0), B, T, H, dk, dv, block_size,
+                                  sfx[0].shape[1], _stream())
+    _lib.check(lib, rc)
+    return outs, d_s0

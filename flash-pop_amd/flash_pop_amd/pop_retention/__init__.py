@@ -5,6 +5,16 @@ Same call signature and returns as the reference's FlashPOPRetention
 the recurrent state after every full block; there is no final-state output.  The block size
 is kept on the autograd context, so T need not be a multiple of it in the backward pass
 (the reference re-derives it as T // num_blocks, pop_retention/__init__.py:39-40).
+
+flash_pop_retention_with_suffixes(q, k, v, s, head_decays, block_size, q_sfx, k_sfx, v_sfx)
+    -> (o, o_sfx, last_state)
+
+One POP layer step in a single walk: what POPDecoderLayer.pop_forward obtains from
+flash_pop_retention followed by fused_chunk_retention on the suffix batch seeded with
+[s, block_states] (flash_pop/pop_retnet.py:107-171), without writing the block states, reading
+them back or concatenating them.  q_sfx, k_sfx, v_sfx are [B * (N + 1), Ls, H, d] with the block
+index fastest (N = T // block_size, T a multiple of block_size, Ls <= 64); last_state is the
+state after the last block, the reference's `states[:, -1]`.
 """
 import torch
 
@@ -35,3 +45,30 @@ class FlashPOPRetention(torch.autograd.Function):
 
 
 flash_pop_retention = FlashPOPRetention.apply
+
+
+class FlashPOPRetentionWithSuffixes(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, q, k, v, s, head_decays, block_size, q_sfx, k_sfx, v_sfx):
+        block_size = int(block_size)
+        assert block_size >= 1, f"block_size must be positive, got {block_size}"
+        q, k, v, s, shape = _ops.prepare(q, k, v, s, head_decays)
+        sfx = _ops.prepare_suffixes(q_sfx, k_sfx, v_sfx, shape, block_size)
+        o, o_sfx, last_state = _ops.pop_fused_fwd(q, k, v, s, sfx, head_decays, block_size, shape)
+        ctx.save_for_backward(q, k, v, s, *sfx)
+        ctx.head_decays = tuple(head_decays)
+        ctx.shape = shape
+        ctx.block_size = block_size
+        return o, o_sfx, last_state
+
+    @staticmethod
+    def backward(ctx, d_o, d_o_sfx, d_last_state):
+        q, k, v, s, *sfx = ctx.saved_tensors
+        want_ds0 = s is not None and ctx.needs_input_grad[3]
+        (dq, dk, dv, dq_s, dk_s, dv_s), d_s0 = _ops.pop_fused_bwd(q, k, v, s, sfx, ctx.head_decays, ctx.block_size,
+                                                                   ctx.shape, d_o, d_o_sfx, d_last_state, want_ds0)
+        return dq, dk, dv, d_s0, None, None, dq_s, dk_s, dv_s
+
+
+flash_pop_retention_with_suffixes = FlashPOPRetentionWithSuffixes.apply

@@ -66,6 +66,32 @@ int fp_pop_retention_bwd(const void* q, const void* k, const void* v, const void
                          const void* d_o, const void* d_block_states, void* dq, void* dk_, void* dv_, void* d_s0,
                          int B, int T, int H, int dk, int dv, int block_size, void* stream);
 
+/* One POP layer step in a single walk over each sequence: the context retention and the N + 1
+ * suffix retentions that POPDecoderLayer.pop_forward runs as two ops, pop_chunkwise and then
+ * _suffixes_forward -> _retention_chunkwise (flash_pop/pop_retnet.py:107/113 and :152-171).
+ * Suffix n of sequence b reads the state at token n * block_size (s0 for n = 0) straight from
+ * the walk; block states are neither written nor read back, and the concatenation of
+ * [s0, block states] (pop_retnet.py:163-165) does not happen.
+ *   q_sfx, k_sfx  [B * (N + 1), sfx_len, H, dk], v_sfx, o_sfx [B * (N + 1), sfx_len, H, dv], block
+ *                 index fastest, N = T / block_size, as the reference batches its suffixes
+ *   s_out         out: state after the last block, the reference's `last_state` (pop_retnet.py:169);
+ *                 may be NULL
+ * Needs T % block_size == 0 (as the reference's layer does), 1 <= sfx_len <= 64 and dk, dv in {64, 128}. */
+int fp_pop_fused_fwd(const void* q, const void* k, const void* v, const void* s0, const void* q_sfx, const void* k_sfx,
+                     const void* v_sfx, const double* head_decays, void* o, void* o_sfx, void* s_out, int B, int T,
+                     int H, int dk, int dv, int block_size, int sfx_len, void* stream);
+
+/* Gradients of fp_pop_fused_fwd (what autograd derives for the reference's two ops plus the
+ * concatenation between them).
+ *   d_o, d_o_sfx  gradients of o and o_sfx
+ *   d_s_out       gradient of s_out, may be NULL (zeros)
+ *   dq .. dv_sfx  out: gradients of q, k, v and of the suffix tensors
+ *   d_s0          out: gradient of s0 (context and suffix 0 together), may be NULL (not wanted) */
+int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0, const void* q_sfx, const void* k_sfx,
+                     const void* v_sfx, const double* head_decays, const void* d_o, const void* d_o_sfx,
+                     const void* d_s_out, void* dq, void* dk_, void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx,
+                     void* d_s0, int B, int T, int H, int dk, int dv, int block_size, int sfx_len, void* stream);
+
 /* Message for the last nonzero return on this thread ("" if none). */
 const char* fp_last_error(void);
 

@@ -9,5 +9,6 @@ from .retention_oracle import (  # noqa: F401
     retention_chunk_grads,
     recurrent_step,
     pop_suffix_retention,
+    pop_fused_retention,
     rms_error_ratio,
 )

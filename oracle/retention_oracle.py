@@ -12,6 +12,7 @@ the benchmark do.  It restates, in plain torch, what the reference computes in
   * flash_pop/retnet.py:70-76                      per-head decay values         -> head_decays
   * flash_pop/retnet.py:79-101                     one-token recurrent step      -> recurrent_step
   * flash_pop/pop_retnet.py:152-171                POP suffix state selection    -> pop_suffix_retention
+  * flash_pop/pop_retnet.py:107,152-171            context + suffixes of one layer -> pop_fused_retention
 
 Conventions carried over from the reference: tensors are [B, T, H, d]; the
 state is [B, H, dk, dv]; the public entry points divide K by sqrt(dk)
@@ -173,6 +174,24 @@ def pop_suffix_retention(q_sfx: Tensor, k_sfx: Tensor, v_sfx: Tensor, state0: Op
     assert q_sfx.shape[0] == B * (N + 1)
     out, _ = chunkwise_retention(q_sfx, k_sfx, v_sfx, starts, decays, chunk_size)
     return out
+
+
+def pop_fused_retention(q: Tensor, k: Tensor, v: Tensor, state0: Optional[Tensor], q_sfx: Tensor, k_sfx: Tensor,
+                        v_sfx: Tensor, decays: Sequence[float], block_size: int):
+    """One POP layer step as the reference composes it (flash_pop/pop_retnet.py:107 then :152-171):
+    the context through the block-state retention, then the N + 1 suffixes per sequence from
+    [state0, block states].  Returns (o, o_sfx, state after the last FULL block), the last being
+    what the reference keeps as the new recurrent state (`last_state = states[:, -1]`, :169); with
+    no full block it is state0 (zeros if None)."""
+    o, block_states = pop_retention(q, k, v, state0, decays, block_size)
+    o_sfx = pop_suffix_retention(q_sfx, k_sfx, v_sfx, state0, block_states, decays)
+    if block_states.shape[1] > 0:
+        last = block_states[:, -1]
+    elif state0 is not None:
+        last = state0
+    else:
+        last = q.new_zeros(q.shape[0], q.shape[2], q.shape[3], v.shape[3])
+    return o, o_sfx, last
 
 
 def rms_error_ratio(approx: Tensor, ref: Tensor) -> float:

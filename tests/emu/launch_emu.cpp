@@ -48,25 +48,35 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
   fpk::PassArgs a = args;
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool ws = a.dA == 64 || a.dA == 128;
+  const bool suffix = a.Ls > 0;
+  if (suffix) {
+    if (!ws || blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > fpk::CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys) {
+      *err = "suffix walk: needs dA of 64 or 128, T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
+      return 1;
+    }
+    a.slots = a.B;
+  }
   // Pretend the chip is tiny, so that the several-entries-per-workgroup path is exercised:
   // at most two workgroups per (head, column tile).
-  if (a.slots <= 0) a.slots = (ws && !blocks && a.B > 2) ? 2 : a.B;
+  if (a.slots <= 0) a.slots = (ws && !blocks && !suffix && a.B > 2) ? 2 : a.B;
   if (a.slots > a.B) a.slots = a.B;
   const bool multi = a.slots < a.B;
-  if (multi && (!ws || blocks)) {
+  if (multi && (!ws || blocks || suffix)) {
     *err = "several batch entries per workgroup need the plain wave-specialised kernel";
     return 1;
   }
   const int nwg = a.slots * a.H * (a.dB / fpk::BV);
   switch (a.dA) {
     case 64:
-      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, true, false>(a, l); });
-      if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, false, true>(a, l); });
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, false, false>(a, l); });
+      if (suffix) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_SUFFIX>(a, l); });
+      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_BLOCKS>(a, l); });
+      if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_MULTI>(a, l); });
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_PLAIN>(a, l); });
     case 128:
-      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, true, false>(a, l); });
-      if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, false, true>(a, l); });
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, false, false>(a, l); });
+      if (suffix) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_SUFFIX>(a, l); });
+      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_BLOCKS>(a, l); });
+      if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_MULTI>(a, l); });
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_PLAIN>(a, l); });
     case 256:
       return run_grid(fpk::NTHREADS, nwg, fpk::lds_bytes(256), [&](char* l) { fpk::retention_pass<256>(a, l); });
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;

@@ -161,3 +161,55 @@ def raw_pop_bwd(lib, q, k, v, s, decays, block, d_o, d_states, stream=None, want
     _check(lib, lib.fp_pop_retention_bwd(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(d_o), _p(dst), _p(dq), _p(dk_),
                                          _p(dv_), _p(ds0), B, T, H, dk, dv, block, stream))
     return dq, dk_, dv_, ds0
+
+
+def make_suffix_inputs(B, nblk, Ls, H, dk, dv, seed=0, device="cpu"):
+    """q_sfx, k_sfx, v_sfx ~ N(0,1) in bf16, [B * (nblk + 1), Ls, H, d], block index fastest."""
+    g = torch.Generator().manual_seed(seed)
+    n = B * (nblk + 1)
+    return tuple(torch.randn(n, Ls, H, d, generator=g).to(BF16).to(device) for d in (dk, dk, dv))
+
+
+def oracle_fused(q, k, v, s, sfx, decays, block, cot=None, dtype=torch.float32):
+    """Oracle for the fused POP step.  cot = (d_o, d_o_sfx, d_s_out or None) adds the autograd
+    gradients w.r.t. (q, k, v, q_sfx, k_sfx, v_sfx, s)."""
+    want = cot is not None
+    leaf = lambda t: None if t is None else t.detach().cpu().to(dtype).requires_grad_(want)
+    q_, k_, v_, s_ = (leaf(t) for t in (q, k, v, s))
+    sf = [leaf(t) for t in sfx]
+    o, o_sfx, last = oracle.pop_fused_retention(q_, k_, v_, s_, *sf, decays, block)
+    if not want:
+        return o, o_sfx, last
+    loss = (o * cot[0].cpu().to(dtype)).sum() + (o_sfx * cot[1].cpu().to(dtype)).sum()
+    if cot[2] is not None:
+        loss = loss + (last * cot[2].cpu().to(dtype)).sum()
+    leaves = [q_, k_, v_, *sf] + ([s_] if s_ is not None else [])
+    grads = list(torch.autograd.grad(loss, leaves))
+    if s_ is None:
+        grads.append(None)
+    return o.detach(), o_sfx.detach(), last.detach(), grads
+
+
+def raw_fused_fwd(lib, q, k, v, s, sfx, decays, block, stream=None, want_state=True):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    Ls = sfx[0].shape[1]
+    nan = lambda *shape: torch.full(shape, float("nan"), dtype=BF16, device=q.device)
+    o, o_sfx = nan(B, T, H, dv), nan(*sfx[2].shape)
+    S = nan(B, H, dk, dv) if want_state else None
+    _check(lib, lib.fp_pop_fused_fwd(_p(q), _p(k), _p(v), _p(s), _p(sfx[0]), _p(sfx[1]), _p(sfx[2]), _dec(decays),
+                                     _p(o), _p(o_sfx), _p(S), B, T, H, dk, dv, block, Ls, stream))
+    return o, o_sfx, S
+
+
+def raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot, stream=None, want_ds0=True):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    Ls = sfx[0].shape[1]
+    nan = lambda t: torch.full(tuple(t.shape), float("nan"), dtype=BF16, device=q.device)
+    outs = [nan(q), nan(k), nan(v), nan(sfx[0]), nan(sfx[1]), nan(sfx[2])]
+    ds0 = torch.full((B, H, dk, dv), float("nan"), dtype=BF16, device=q.device) if want_ds0 else None
+    _check(lib, lib.fp_pop_fused_bwd(_p(q), _p(k), _p(v), _p(s), _p(sfx[0]), _p(sfx[1]), _p(sfx[2]), _dec(decays),
+                                     _p(cot[0]), _p(cot[1]), _p(cot[2]), *[_p(t) for t in outs], _p(ds0),
+                                     B, T, H, dk, dv, block, Ls, stream))
+    return outs + [ds0]

@@ -64,6 +64,28 @@ def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
                 ("ds0", ds0, gs)])
 
 
+FUSED_NAMES = ("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0")
+
+
+@pytest.mark.parametrize("B,nblk,block,Ls,H,dk,dv,state_std", [
+    (1, 2, 64, 16, 2, 128, 128, 0.5),    # block == chunk
+    (2, 2, 80, 5, 1, 64, 128, None),     # block of a full and a short chunk, no initial state
+    (1, 3, 24, 64, 1, 128, 64, 0.5),     # block shorter than a chunk, suffix as long as one
+    (1, 1, 130, 1, 1, 64, 64, 0.0),      # one block of three chunks, one-token suffixes
+])
+def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std):
+    decays = oracle.head_decays(H, (4, 9))
+    T = nblk * block
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + Ls, state_std=state_std)
+    sfx = hp.make_suffix_inputs(B, nblk, Ls, H, dk, dv, seed=T + Ls + 1)
+    cot = hp.make_cotangents([(B, T, H, dv), tuple(sfx[2].shape), (B, H, dk, dv)], seed=T + 2)
+    o, o_sfx, S = hp.raw_fused_fwd(emu_lib, q, k, v, s, sfx, decays, block)
+    grads = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
+    o_ref, os_ref, S_ref, g_ref = hp.oracle_fused(q, k, v, s, sfx, decays, block, cot)
+    _check_all([("o", o, o_ref), ("o_sfx", o_sfx, os_ref), ("s_out", S, S_ref)])
+    _check_all([(n, g, r) for n, g, r in zip(FUSED_NAMES, grads, g_ref)])
+
+
 def test_optional_outputs_and_determinism(emu_lib):
     decays = oracle.head_decays(2)
     q, k, v, s = hp.make_inputs(1, 90, 2, 64, 64, seed=3, state_std=0.5)

@@ -1,0 +1,125 @@
+"""GPU parity tests for flash_pop_retention_with_suffixes (context + suffixes in one walk),
+through the autograd Function and the C ABI.  The oracle composes the two steps the way the
+reference's layer does.  Same bar as test_retention_gpu.py."""
+import pytest
+import torch
+
+import helpers as hp
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+GRADS = ("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0")
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, oracle_batches=None, d_last=True):
+    from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
+    T = N * block
+    _say(f"[fused pop] B{B} N{N} block{block} Ls{Ls} H{H} dk{dk} dv{dv} s0={state_std} seed={seed}")
+    decays = oracle.head_decays(H, decay_range)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=seed, state_std=state_std)
+    sfx = hp.make_suffix_inputs(B, N, Ls, H, dk, dv, seed=seed + 1)
+    cot = hp.make_cotangents([(B, T, H, dv), tuple(sfx[2].shape), (B, H, dk, dv)], seed=seed + 2)
+    if not d_last:
+        cot[2] = None
+    ctx = [None if t is None else t.to(DEV).requires_grad_() for t in (q, k, v, s)]
+    sx = [t.to(DEV).requires_grad_() for t in sfx]
+    o, o_sfx, last = flash_pop_retention_with_suffixes(*ctx, decays, block, *sx)
+    outs, cots = [o, o_sfx], [cot[0].to(DEV), cot[1].to(DEV)]
+    if d_last:
+        outs.append(last)
+        cots.append(cot[2].to(DEV))
+    torch.autograd.backward(outs, cots)
+    torch.cuda.synchronize()
+    for b in (range(B) if oracle_batches is None else oracle_batches):
+        sl, ssl = slice(b, b + 1), slice(b * (N + 1), (b + 1) * (N + 1))
+        cut = lambda t, w: None if t is None else t[w]
+        o_ref, os_ref, last_ref, g_ref = hp.oracle_fused(
+            q[sl], k[sl], v[sl], cut(s, sl), [t[ssl] for t in sfx], decays, block,
+            (cot[0][sl], cot[1][ssl], cut(cot[2], sl)))
+        hp.assert_close(o[sl], o_ref, f"o[b={b}]", head_dim=2)
+        hp.assert_close(o_sfx[ssl], os_ref, f"o_sfx[b={b}]", head_dim=2)
+        hp.assert_close(last[sl], last_ref, f"last_state[b={b}]", head_dim=1)
+        leaves = ctx[:3] + sx + [ctx[3]]
+        for name, leaf, ref in zip(GRADS, leaves, g_ref):
+            if ref is None:
+                continue
+            w = sl if "sfx" not in name else ssl
+            hp.assert_close(leaf.grad[w], ref, f"{name}[b={b}]", head_dim=1 if name == "ds0" else 2)
+    return o, o_sfx, last
+
+
+@pytest.mark.parametrize("B,N,block,Ls,H,dk,dv", [
+    (2, 4, 64, 16, 4, 128, 128),     # block == chunk, headline head dims
+    (2, 3, 144, 16, 4, 64, 128),     # reference generation block size: two full chunks and a short one
+    (3, 5, 15, 7, 2, 64, 64),        # block and suffix shorter than a chunk
+    (1, 2, 256, 64, 2, 128, 64),     # suffix as long as a chunk
+    (2, 8, 32, 1, 2, 64, 128),       # one-token suffixes
+])
+def test_fused_parity_sweep(B, N, block, Ls, H, dk, dv):
+    run_fused(B, N, block, Ls, H, dk, dv, 0.3, seed=N * block + Ls, decay_range=(5, 12))
+
+
+def test_fused_without_state_and_without_last_state_gradient():
+    run_fused(2, 3, 64, 8, 2, 64, 64, None, seed=5)
+    run_fused(1, 2, 96, 8, 2, 128, 128, 0.2, seed=6, d_last=False)
+
+
+def test_fused_matches_the_two_op_path():
+    """Context outputs are bit-identical to flash_pop_retention's when block is a chunk multiple
+    (same partition, same arithmetic); suffix outputs agree with the two-op path to the parity bar
+    (there the block states pass through bf16 on the way)."""
+    from flash_pop_amd import flash_pop_retention, fused_chunk_retention
+    from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
+    B, N, block, Ls, H, d = 2, 6, 128, 16, 4, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, N * block, H, d, d, seed=61, state_std=0.1, device=DEV)
+    sfx = hp.make_suffix_inputs(B, N, Ls, H, d, d, seed=62, device=DEV)
+    o, o_sfx, last = flash_pop_retention_with_suffixes(q, k, v, s, decays, block, *sfx)
+    o2, states = flash_pop_retention(q, k, v, s, decays, block)
+    starts = torch.cat((s[:, None], states), dim=1).flatten(0, 1)
+    o_sfx2, _ = fused_chunk_retention(*sfx, starts, decays)
+    assert torch.equal(o, o2) and torch.equal(last, states[:, -1])
+    hp.assert_close(o_sfx, o_sfx2.float(), "o_sfx vs two-op path", head_dim=2)
+
+
+def test_fused_raw_abi_optional_outputs():
+    """s_out and d_s0 may be NULL; the other outputs do not change."""
+    from flash_pop_amd import _lib
+    lib = _lib.load()
+    B, N, block, Ls, H, d = 1, 2, 64, 16, 2, 64
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, N * block, H, d, d, seed=71, state_std=0.3, device=DEV)
+    sfx = hp.make_suffix_inputs(B, N, Ls, H, d, d, seed=72, device=DEV)
+    cot = hp.make_cotangents([(B, N * block, H, d), tuple(sfx[2].shape), (B, H, d, d)], seed=73, device=DEV)
+    a = hp.raw_fused_fwd(lib, q, k, v, s, sfx, decays, block)
+    b = hp.raw_fused_fwd(lib, q, k, v, s, sfx, decays, block, want_state=False)
+    ga = hp.raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot)
+    gb = hp.raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot, want_ds0=False)
+    torch.cuda.synchronize()
+    assert b[2] is None and torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert gb[6] is None and all(torch.equal(x, y) for x, y in zip(ga[:6], gb[:6]))
+
+
+def test_fused_argument_errors():
+    from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
+    decays = oracle.head_decays(2)
+    q, k, v, s = hp.make_inputs(1, 128, 2, 64, 64, seed=1, state_std=0.1, device=DEV)
+    sfx = hp.make_suffix_inputs(1, 2, 8, 2, 64, 64, seed=2, device=DEV)
+    with pytest.raises(ValueError, match="multiple of block_size"):
+        flash_pop_retention_with_suffixes(q, k, v, s, decays, 50, *sfx)
+    with pytest.raises(ValueError, match="one additional suffix block"):
+        flash_pop_retention_with_suffixes(q, k, v, s, decays, 32, *sfx)
+    long_sfx = hp.make_suffix_inputs(1, 2, 65, 2, 64, 64, seed=3, device=DEV)
+    with pytest.raises(RuntimeError, match="suffix length"):
+        flash_pop_retention_with_suffixes(q, k, v, s, decays, 64, *long_sfx)
+
+
+def test_config4_fused():
+    """BASELINE config 4 in one walk: B8 H16 d128, T4096 in 64-token blocks, 65 suffixes of 16 tokens
+    per sequence.  Oracle on one sequence."""
+    run_fused(8, 64, 64, 16, 16, 128, 128, 0.05, seed=40, oracle_batches=[5])

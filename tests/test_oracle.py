@@ -221,6 +221,29 @@ def test_pop_suffix_equals_concatenated_context():
     assert torch.equal(got0, gotz)
 
 
+def test_pop_fused_is_the_composition_and_pins_last_state():
+    decays = (0.9, 0.97)
+    B, N, bs, Ls, H, dk, dv = 2, 3, 5, 4, 2, 4, 3
+    for T in (N * bs, N * bs + 2):          # with and without a ragged tail after the last block
+        q, k, v, s = rand_inputs(B, T, H, dk, dv, seed=31)
+        qs, ks, vs, _ = rand_inputs(B * (N + 1), Ls, H, dk, dv, False, seed=32)
+        o, o_sfx, last = oracle.pop_fused_retention(q, k, v, s, qs, ks, vs, decays, bs)
+        o_cf, _ = closed_form(q, k, v, s, decays)
+        _, S_blocks = closed_form(q[:, :N * bs], k[:, :N * bs], v[:, :N * bs], s, decays)
+        assert torch.allclose(o, o_cf, atol=1e-10) and torch.allclose(last, S_blocks, atol=1e-10)
+        for b in range(B):
+            for n in range(N + 1):
+                i = b * (N + 1) + n
+                cat = lambda ctx, sfx: torch.cat((ctx[b:b + 1, :n * bs], sfx[i:i + 1]), dim=1)
+                ref, _ = closed_form(cat(q, qs), cat(k, ks), cat(v, vs), s[b:b + 1], decays)
+                assert torch.allclose(o_sfx[i], ref[0, n * bs:], atol=1e-10)
+    # no full block: the last state is the initial one
+    q, k, v, s = rand_inputs(1, 3, 2, 4, 3, seed=33)
+    qs, ks, vs, _ = rand_inputs(1, 2, 2, 4, 3, False, seed=34)
+    _, _, last = oracle.pop_fused_retention(q, k, v, s, qs, ks, vs, decays, 5)
+    assert torch.equal(last, s)
+
+
 def test_fp32_matches_fp64_at_config1():
     """BASELINE config 1 (fp32, B1 H4 T512 d64, chunk 64, no initial state): the fp32 oracle
     is within 1e-4 of the float64 closed form."""
