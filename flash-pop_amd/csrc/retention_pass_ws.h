@@ -53,7 +53,7 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 // WALK_SUFFIX  a suffix of p.Ls tokens hangs off every block boundary (positions 0, block, ...,
 //              T; T is a multiple of the block size).  It is one more item of the walk, placed at
 //              its boundary, with its own tensors: it reads the state at the boundary without
-//              advancing it.  Walking forward its keys get weight 0 and R is not decayed; walking
+//              advancing it.  Walking forward its keys stay out of R and R is not decayed; walking
 //              backward its read-out weight is 0 and what it adds to R (the gradient of the state
 //              it read) is not decayed either.
 enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3 };
@@ -588,16 +588,15 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   int Lk_cached = -1;
   float wkey[4];
   auto store_transposed = [&](const ChunkRegs& cr, const Chunk& ck) {
-    const bool sf = SFX && ck.sfx;
-    const int key = ck.L + (sf ? 256 : 0);
-    if (key != Lk_cached) {
-      Lk_cached = key;
+    if (SFX && ck.sfx && !rev) return;   // walking forward, a suffix's keys never enter the state
+    if (ck.L != Lk_cached) {
+      Lk_cached = ck.L;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int j = 4 * w_tg + r;
         int e = rev ? (j + 1) : (ck.L - 1 - j);
         if (e < 0) e = 0;
-        wkey[r] = (sf && !rev) ? 0.f : p.s_update * fprt::exp2_approx((float)e * lg);
+        wkey[r] = p.s_update * fprt::exp2_approx((float)e * lg);
       }
     }
 #pragma unroll
@@ -660,9 +659,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       nxt = nn;
       return true;
     }
+    // A suffix carries tokens only in its first k-steps, and none that enter the state when
+    // walking forward: the other k-steps are skipped (uniform branches).
+    const bool sfx_item = SFX && cur.sfx;
+    const int nk = sfx_item ? (rev ? (cur.L + 15) >> 4 : 0) : 4;
+
     // ---- phase 0: request the operands of the state update (this wave's whole W^T slab, the
     // first half of Z^T); decay R while they arrive
-    const int gkey = (SFX && cur.sfx) ? 0 : cur.L;   // a suffix does not advance the state
+    const int gkey = sfx_item ? 0 : cur.L;   // a suffix does not advance the state
     if (gkey != Lg_cached) {
       Lg_cached = gkey;
       gL = fprt::exp2_approx((float)gkey * lg);
@@ -670,16 +674,22 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const uint16_t* zt = ZT + s * BV * T_LD;
     u32x4 wf[4], zlo[NNW][2], zhi[NNW][2];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) wf[kt] = ld_token_frag(wt + c * T_LD + 16 * kt + 4 * g);
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-      for (int nq = 0; nq < NNW; ++nq) zlo[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * kt + 4 * g);
+    for (int kt = 0; kt < 4; ++kt) {
+      if (kt < nk) wf[kt] = ld_token_frag(wt + c * T_LD + 16 * kt + 4 * g);
     }
 #pragma unroll
-    for (int nq = 0; nq < NNW; ++nq) {
+    for (int kt = 0; kt < 2; ++kt) {
+      if (kt < nk) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) racc[nq][r] *= gL;
+        for (int nq = 0; nq < NNW; ++nq) zlo[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * kt + 4 * g);
+      }
+    }
+    if (!sfx_item) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) racc[nq][r] *= gL;
+      }
     }
     fprt::sched_fence();
     fprt::prof_stamp(it, 1);
@@ -688,14 +698,18 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // requested and the W of chunk it + 1 (zeros if there is none) is transposed.  The W^T slab is overwritten only after all of it was read.
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
+      if (kt < nk) {
 #pragma unroll
-      for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[kt], zlo[nq][kt], racc[nq]);
+        for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[kt], zlo[nq][kt], racc[nq]);
+      }
     }
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
+      if (2 + kt < nk) {
 #pragma unroll
-      for (int nq = 0; nq < NNW; ++nq)
-        zhi[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * (2 + kt) + 4 * g);
+        for (int nq = 0; nq < NNW; ++nq)
+          zhi[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * (2 + kt) + 4 * g);
+      }
     }
     store_transposed(ready, nxt);
     fprt::sched_fence();
@@ -704,8 +718,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // ---- phase 2: second half of the state update; the row-major copies go out in its shadow
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
+      if (2 + kt < nk) {
 #pragma unroll
-      for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc[nq]);
+        for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc[nq]);
+      }
     }
     store_rowmajor(ready, s ^ 1);
     if (!DEEP) prefetch(refill, nn);   // refill and ready are the same set here
