@@ -1,5 +1,5 @@
 #!/bin/bash
-# Collects the rocprofv3 evidence for the pass kernel on BASELINE config 2 (run from the repo
+# Collects the rocprofv3 evidence for the pass kernels on BASELINE configs 2 and 4 (run from the repo
 # root on a GPU box): kernel-trace statistics, then hardware counters in separate passes (one
 # counter group per run), then the same HBM counters on a plain copy of known size for scaling.
 # Raw output goes to gpurun_out/profile/; the figures are summarised by hand into profiles/.
@@ -8,7 +8,7 @@ R=$(cd "$(dirname "$0")/.." && pwd)
 O=$R/gpurun_out/profile
 mkdir -p "$O"
 cd /tmp && export TMPDIR=/tmp
-BENCH="python3 $R/bench.py --steps 5 --warmup 2 --no-cpu --no-pop"
+BENCH="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu"
 COPY="python3 $R/bench.py --copy-calibration"
 run() { name=$1; shift; timeout -s KILL 120 rocprofv3 "$@" --output-format csv -d "$O/$name" -o r -- $CMD > "$O/$name.log" 2>&1; }
 CMD=$BENCH run trace --kernel-trace --stats
