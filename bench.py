@@ -6,7 +6,7 @@ resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic F
 (dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the pass kernel measured
 with events on the launch stream, and the CPU oracle timed on the host cores beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop] [--no-long]
 """
 import argparse
 import json
@@ -169,6 +169,40 @@ def gpu_leg(args):
                 "cost_per_token_vs_plain": ratio(pop_ms),
             },
         }
+    if not args.no_long:
+        # Long context, few streams (config 3): B=2 H=8 T=16384 dk=128 dv=256 with a carried state and
+        # its gradient.  16 streams cannot fill 256 compute units, so the op cuts each sequence into
+        # segments (fp_retention_*_split).
+        del leaves, q, k, v
+        B3, T3, H3, dk3, dv3 = 2, 16384, 8, 128, 256
+        dec3 = oracle.head_decays(H3)
+        q3, k3, v3, s3 = hp.make_inputs(B3, T3, H3, dk3, dv3, seed=4, state_std=0.02, device=dev)
+        d_o3, d_s3 = hp.make_cotangents([(B3, T3, H3, dv3), (B3, H3, dk3, dv3)], seed=5, device=dev)
+        l3 = [t.requires_grad_() for t in (q3, k3, v3, s3)]
+
+        def long_step():
+            o, S = fused_chunk_retention(*l3, dec3)
+            return torch.autograd.grad([o, S], l3, [d_o3, d_s3])
+
+        for _ in range(max(2, args.warmup // 4)):
+            long_step()
+        torch.cuda.synchronize()
+        n = max(3, args.steps // 4)
+        t0 = time.perf_counter()
+        for _ in range(n):
+            long_step()
+        torch.cuda.synchronize()
+        long_ms = (time.perf_counter() - t0) * 1e3 / n
+        f3 = sum(algorithmic_flops(B3, T3, H3, dk3, dv3))
+        b3 = sum(algorithmic_bytes(B3, T3, H3, dk3, dv3))
+        out["long_context"] = {
+            "workload": "config 3: B=2 H=8 T=16384 dk=128 dv=256, carried state, fwd+bwd incl. dS0",
+            "ms_per_step": round(long_ms, 4),
+            "tflops": round(f3 / (long_ms * 1e-3) / 1e12, 2),
+            "algorithmic_gbs": round(b3 / (long_ms * 1e-3) / 1e9, 1),
+            "segments_per_sequence": _lib.load().fp_retention_workspace_bytes(B3, T3, H3, dk3, dv3)
+            // (4 * B3 * H3 * dk3 * dv3),
+        }
     return out
 
 
@@ -211,6 +245,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
+    ap.add_argument("--no-long", action="store_true", help="skip the long-context (config 3) timing")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy (scales the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()

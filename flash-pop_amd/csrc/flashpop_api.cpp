@@ -18,6 +18,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <cstdint>
 
 #include "pass_args.h"
 
@@ -142,6 +143,142 @@ int backward(const Shape& s, const void* q, const void* k, const void* v, const 
   return run(a, stream, "dv");
 }
 
+// ---- long sequences, few streams: cut every sequence into segments ---------------------------
+// One workgroup walks one (batch, head, column tile) stream from end to end, so B * H * tiles
+// workgroups is all the parallelism a pass has.  When that leaves most of the chip idle, each
+// sequence is cut into S equal segments that run as separate sequences:
+//   1. a state-only pass gives the state each segment contributes on its own,
+//   2. a scan over the S contributions gives the state at the start of every segment,
+//   3. the ordinary pass runs on B * S sequences from those states.
+// The backward does the same for S (needed by the dq pass; recomputed, not stored) and, walking
+// backward, for dS.  Segment states pass through bf16 like POP block states do.
+
+// Number of segments per sequence (1: do not cut) for a call whose narrowest pass has
+// `tiles` column tiles per stream.  Cutting costs an extra state-only pass per recurrence, so it
+// is done only when the uncut call would leave at least two thirds of the compute units idle.
+int plan_segments(const Shape& s, int tiles) {
+  constexpr int kMinChunks = 4;                 // shortest segment worth a workgroup of its own
+  if (s.dk > 128) return 1;                     // the state-only walk needs dA = dk of 64 or 128
+  if (s.T % fpk::CH != 0) return 1;
+  const int chunks = s.T / fpk::CH;
+  const long long streams = (long long)s.B * s.H * tiles;
+  const long long target = fpk_compute_units() / streams;   // segments that fill the chip once
+  if (target < 3) return 1;
+  int best = 1;
+  for (int n = 2; n <= target && n <= chunks; ++n) {
+    if (chunks % n == 0 && chunks / n >= kMinChunks) best = n;
+  }
+  return best;
+}
+int plan_forward(const Shape& s) { return plan_segments(s, s.dv / fpk::BV); }
+int plan_backward(const Shape& s) { return plan_segments(s, (s.dk < s.dv ? s.dk : s.dv) / fpk::BV); }
+
+size_t workspace_bytes(const Shape& s, int segments) {
+  return segments > 1 ? 2 * sizeof(uint16_t) * (size_t)s.B * segments * s.H * s.dk * s.dv : 0;
+}
+
+struct Workspace {
+  uint16_t* contrib;   // [B, S, H, dk, dv]: what each segment adds on its own
+  uint16_t* start;     // [B, S, H, dk, dv]: state at the segment's first token (last, walking backward)
+};
+
+Workspace carve(void* workspace, const Shape& s, int segments) {
+  uint16_t* base = static_cast<uint16_t*>(workspace);
+  return Workspace{base, base + (size_t)s.B * segments * s.H * s.dk * s.dv};
+}
+
+int scan(const Shape& s, int segments, const double* decays, const Workspace& w, const void* r0, void* fin, int reverse,
+         void* stream) {
+  fpk::ScanArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.U = w.contrib; a.R0 = in(r0); a.init = w.start; a.fin = out(fin);
+  a.B = s.B; a.S = segments; a.H = s.H; a.M = s.dk * s.dv; a.Tseg = s.T / segments; a.reverse = reverse;
+  for (int h = 0; h < s.H; ++h) a.log2g[h] = (float)std::log2(decays[h]);
+  const char* msg = "";
+  if (fpk_launch_scan(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "segment scan: %s", msg);
+  return FP_OK;
+}
+
+// the B * S sequences of T / S tokens that the segments form (the same memory, reinterpreted)
+Shape segment_shape(const Shape& s, int segments) { return Shape{s.B * segments, s.T / segments, s.H, s.dk, s.dv}; }
+
+// State-only pass: contributions of the segments to S (forward walk over k, v) or to dS
+// (backward walk over q, dO).
+int contributions(const Shape& seg, const double* decays, const void* w_rows, const void* z_rows, int reverse,
+                  const Workspace& w, void* stream) {
+  fpk::PassArgs a;
+  fill_common(a, seg, decays);
+  const float sc = 1.0f / std::sqrt((float)seg.dk);
+  a.X = in(w_rows);   // never read
+  a.W = in(w_rows); a.Z = in(z_rows);
+  a.Rout = w.contrib;
+  plain_state(a, seg);
+  a.reverse = reverse;
+  a.state_only = 1;
+  a.s_intra = sc; a.s_read = reverse ? sc : 1.f; a.s_update = reverse ? 1.f : sc;
+  return run(a, stream, reverse ? "dS contributions" : "S contributions");
+}
+
+int forward_split(const Shape& s, int segments, const void* q, const void* k, const void* v, const void* s0,
+                  const double* decays, void* o, void* s_out, void* workspace, void* stream) {
+  const Shape seg = segment_shape(s, segments);
+  const Workspace w = carve(workspace, s, segments);
+  int rc;
+  if ((rc = contributions(seg, decays, k, v, 0, w, stream)) != FP_OK) return rc;
+  if ((rc = scan(s, segments, decays, w, s0, s_out, 0, stream)) != FP_OK) return rc;
+  return forward(seg, q, k, v, w.start, decays, o, nullptr, nullptr, 0, stream);
+}
+
+int backward_split(const Shape& s, int segments, const void* q, const void* k, const void* v, const void* s0,
+                   const double* decays, const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_,
+                   void* d_s0, void* workspace, void* stream) {
+  const Shape seg = segment_shape(s, segments);
+  const Workspace w = carve(workspace, s, segments);
+  const float sc = 1.0f / std::sqrt((float)s.dk);
+  fpk::PassArgs a;
+  int rc;
+
+  // S at the start of every segment, then dq
+  if ((rc = contributions(seg, decays, k, v, 0, w, stream)) != FP_OK) return rc;
+  if ((rc = scan(s, segments, decays, w, s0, nullptr, 0, stream)) != FP_OK) return rc;
+  fill_common(a, seg, decays);
+  a.X = in(d_o); a.W = in(v); a.Z = in(k); a.Y = out(dq);
+  a.R0 = w.start;
+  transposed_state(a, seg);
+  a.reverse = 0;
+  a.s_intra = sc; a.s_read = 1.f; a.s_update = sc;
+  if ((rc = run(a, stream, "dq")) != FP_OK) return rc;
+
+  // dS at the end of every segment (the workspace is free again: the stream orders the passes), then dk and dv
+  if ((rc = contributions(seg, decays, q, d_o, 1, w, stream)) != FP_OK) return rc;
+  if ((rc = scan(s, segments, decays, w, d_s_out, d_s0, 1, stream)) != FP_OK) return rc;
+  fill_common(a, seg, decays);
+  a.X = in(v); a.W = in(d_o); a.Z = in(q); a.Y = out(dk_);
+  a.R0 = w.start;
+  transposed_state(a, seg);
+  a.reverse = 1;
+  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
+  if ((rc = run(a, stream, "dk")) != FP_OK) return rc;
+
+  fill_common(a, seg, decays);
+  a.X = in(k); a.W = in(q); a.Z = in(d_o); a.Y = out(dv_);
+  a.R0 = w.start;
+  plain_state(a, seg);
+  a.reverse = 1;
+  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
+  return run(a, stream, "dv");
+}
+
+int check_workspace(const Shape& s, int segments, const void* workspace, size_t bytes) {
+  if (segments <= 1) return FP_OK;
+  if (!workspace) return fail(FP_ERR_NULL_POINTER, "workspace is NULL but fp_retention_workspace_bytes() is nonzero for this shape");
+  if (bytes < workspace_bytes(s, segments))
+    return fail(FP_ERR_BAD_SHAPE, "workspace of %zu bytes is smaller than the %zu that fp_retention_workspace_bytes() asks for",
+                bytes, workspace_bytes(s, segments));
+  if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return fail(FP_ERR_BAD_SHAPE, "workspace must be 16-byte aligned");
+  return FP_OK;
+}
+
 // Suffix tensors of one fused POP call, in the roles q, k, v / d_o (inputs) and o / dq, dk, dv (outputs)
 struct Suffixes {
   const void *q, *k, *v;
@@ -238,6 +375,38 @@ int fp_retention_bwd(const void* q, const void* k, const void* v, const void* s0
   return backward(s, q, k, v, s0, head_decays, d_o, d_s_out, nullptr, 0, dq, dk_, dv_, d_s0, stream);
 }
 
+size_t fp_retention_workspace_bytes(int B, int T, int H, int dk, int dv) {
+  const Shape s{B, T, H, dk, dv};
+  if (B < 1 || T < 1 || H < 1 || H > fpk::MAX_HEADS || !dim_ok(dk) || !dim_ok(dv)) return 0;
+  const int fwd = plan_forward(s), bwd = plan_backward(s);
+  return workspace_bytes(s, fwd > bwd ? fwd : bwd);
+}
+
+int fp_retention_fwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                           void* o, void* s_out, int B, int T, int H, int dk, int dv, void* workspace,
+                           size_t workspace_bytes_given, void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
+  const int segments = plan_forward(s);
+  if (int rc = check_workspace(s, segments, workspace, workspace_bytes_given)) return rc;
+  if (segments <= 1) return forward(s, q, k, v, s0, head_decays, o, s_out, nullptr, 0, stream);
+  return forward_split(s, segments, q, k, v, s0, head_decays, o, s_out, workspace, stream);
+}
+
+int fp_retention_bwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                           const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B,
+                           int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes_given, void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
+    return fail(FP_ERR_NULL_POINTER, "q, k, v, d_o, dq, dk and dv must not be NULL");
+  const int segments = plan_backward(s);
+  if (int rc = check_workspace(s, segments, workspace, workspace_bytes_given)) return rc;
+  if (segments <= 1) return backward(s, q, k, v, s0, head_decays, d_o, d_s_out, nullptr, 0, dq, dk_, dv_, d_s0, stream);
+  return backward_split(s, segments, q, k, v, s0, head_decays, d_o, d_s_out, dq, dk_, dv_, d_s0, workspace, stream);
+}
+
 int fp_pop_retention_fwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
                          void* o, void* block_states, int B, int T, int H, int dk, int dv, int block_size,
                          void* stream) {
@@ -290,6 +459,6 @@ int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0
 
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1001; }
+int fp_version(void) { return 1002; }
 
 }  // extern "C"

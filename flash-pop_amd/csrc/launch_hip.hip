@@ -2,6 +2,7 @@
 #include "device_rt.h"
 #include "retention_pass.h"
 #include "retention_pass_ws.h"
+#include "segment_scan.h"
 
 namespace {
 
@@ -17,6 +18,10 @@ template <int DA>
 __global__ __launch_bounds__(fpk::NTHREADS) void retention_pass_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   fpk::retention_pass<DA>(args, lds);
+}
+
+__global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
+  fpk::segment_scan(args);
 }
 
 template <typename Kernel>
@@ -61,7 +66,7 @@ extern "C" int fpk_dbg_set(int flags) {
 #endif
 
 // Compute units of the current device (cached per thread and device).
-static int compute_units() {
+int fpk_compute_units() {
   static thread_local int dev_cached = -1, cus = 0;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -74,7 +79,7 @@ static int compute_units() {
 
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  static thread_local int armed[9] = {-1, -1, -1, -1, -1, -1, -1, -1, -1};
+  static thread_local int armed[11] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
   fpk::PassArgs a = args;
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool ws = a.dA == 64 || a.dA == 128;
@@ -94,13 +99,17 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
     a.slots = a.B;
     if (ws && !blocks && !suffix) {
       const int per_slot = a.H * (a.dB / fpk::BV);
-      int fit = compute_units() / per_slot;
+      int fit = fpk_compute_units() / per_slot;
       if (fit < 1) fit = 1;
       if (fit < a.B) a.slots = fit;
     }
   }
   if (a.slots > a.B) a.slots = a.B;
   const bool multi = a.slots < a.B;
+  if (a.state_only && (!ws || blocks || suffix || !a.Rout)) {
+    *err = "state-only walk: needs dA of 64 or 128, a final-state buffer, no block states and no suffixes";
+    return 1;
+  }
   if (multi && (!ws || blocks || suffix)) {
     *err = "several batch entries per workgroup need the plain wave-specialised kernel";
     return 1;
@@ -109,15 +118,38 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
     case 64:
       if (suffix) return launch(retention_pass_ws_kernel<64, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[7], a, s, err);
       if (blocks) return launch(retention_pass_ws_kernel<64, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
+      if (a.state_only) return launch(retention_pass_ws_kernel<64, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[9], a, s, err);
       if (multi) return launch(retention_pass_ws_kernel<64, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
       return launch(retention_pass_ws_kernel<64, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[2], a, s, err);
     case 128:
       if (suffix) return launch(retention_pass_ws_kernel<128, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[8], a, s, err);
       if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
+      if (a.state_only) return launch(retention_pass_ws_kernel<128, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[10], a, s, err);
       if (multi) return launch(retention_pass_ws_kernel<128, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[4], a, s, err);
       return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[5], a, s, err);
     case 256:
       return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[6], a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
+}
+
+int fpk_launch_scan(const fpk::ScanArgs& a, void* stream, const char** err) {
+  if (a.M % fpk::SCAN_VEC != 0 || a.B < 1 || a.S < 1 || a.H < 1 || !a.U || !a.init) {
+    *err = "segment scan: bad arguments";
+    return 1;
+  }
+  const long long items = (long long)a.B * a.H * (a.M / fpk::SCAN_VEC);
+  const long long blocks = (items + fpk::SCAN_THREADS - 1) / fpk::SCAN_THREADS;
+  if (blocks > 0x7fffffffLL) {
+    *err = "segment scan: too many state matrices";
+    return 1;
+  }
+  hipLaunchKernelGGL(segment_scan_kernel, dim3((unsigned)blocks), dim3(fpk::SCAN_THREADS), 0,
+                     static_cast<hipStream_t>(stream), a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    *err = hipGetErrorString(e);
+    return 1;
+  }
+  return 0;
 }

@@ -45,6 +45,7 @@ struct PassArgs {
   int block;             // block size in tokens; chunks never straddle a multiple of it (0: none)
   int reverse;
   int Ls;                // tokens per suffix, 1..CH; 0: no suffixes
+  int state_only;        // only R is wanted (Rout per sequence): X is not read, Y not written, no read-out
   int slots;             // workgroups per (head, column tile); workgroup `slot` walks the batch entries
                          // slot, slot + slots, ... one after another.  0: the launcher chooses.
   float s_intra, s_read, s_update;
@@ -60,8 +61,31 @@ constexpr int lds_bytes(int dA) {
               + CH * (BV + 8));      // Y staging
 }
 
+// Arguments of the segment scan that stitches a sequence cut into S segments back together.
+// U[b][s] is the state a segment contributes on its own (zero initial state); with g = gamma^Tseg
+//   init[b][0] = R0[b] (zeros if null),  init[b][s] = g init[b][s-1] + U[b][s-1],
+//   fin[b] = g init[b][S-1] + U[b][S-1]
+// `reverse` runs the same recurrence from the last segment to the first (state gradients).
+// All matrices are bf16, M = dk * dv elements each, laid out [B, S, H, M] (U, init) and [B, H, M].
+struct ScanArgs {
+  const uint16_t* U;
+  const uint16_t* R0;   // nullable
+  uint16_t* init;
+  uint16_t* fin;        // nullable
+  int B, S, H, M, Tseg, reverse;
+  float log2g[MAX_HEADS];
+};
+constexpr int SCAN_THREADS = 256;
+constexpr int SCAN_VEC = 8;   // elements per thread
+
 }  // namespace fpk
 
 // Launches the pass kernel on `stream` (a hipStream_t, or ignored by the CPU test harness).
 // Returns 0 on success; on failure returns nonzero and *err points at a static message.
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err);
+
+// Launches the segment scan.  Same conventions as fpk_launch_pass.
+int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);
+
+// Compute units of the current device (what the launcher sizes its grids against).
+int fpk_compute_units();

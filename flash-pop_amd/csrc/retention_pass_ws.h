@@ -56,12 +56,15 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 //              advancing it.  Walking forward its keys stay out of R and R is not decayed; walking
 //              backward its read-out weight is 0 and what it adds to R (the gradient of the state
 //              it read) is not decayed either.
-enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3 };
+// WALK_STATE   like WALK_MULTI, but only the final R of every sequence is wanted (p.state_only):
+//              the readout waves feed Z and do nothing else, X is not read and Y not written.
+enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WALK_STATE = 4 };
 
 template <int DA, int MODE>
 FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
-  constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI, SFX = MODE == WALK_SUFFIX;
+  constexpr bool STATE = MODE == WALK_STATE;
+  constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI || STATE, SFX = MODE == WALK_SUFFIX;
   constexpr int X_LD = DA + 8;
   constexpr int T_LD = CH + 4;      // row length of the transposed tiles (tokens)
   constexpr int RT_LD = DA + 8;
@@ -248,7 +251,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     };
     auto feed_load = [&](FeedRegs& fr, const Chunk& c2) {
       const bool live = c2.ok && !(dbg & 1);
-      const uint32_t lenA = live ? (uint32_t)(c2.L - 1) * rowA + p.dA * 2 : 0u;
+      const uint32_t lenA = (live && !STATE) ? (uint32_t)(c2.L - 1) * rowA + p.dA * 2 : 0u;
       const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
       const bool sf = SFX && c2.sfx;
       const fprt::BufView xv = fprt::make_buf((sf ? Xsg : Xg) + (live ? rowsA(c2) : 0), lenA);
@@ -283,8 +286,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     auto drain_y = [&](const Chunk& c2, int s) {
       const uint16_t* src = YB + s * CH * YB_LD + y_row * YB_LD + y_col;
       const u32x4 v0 = ld128(src), v1 = ld128(src + 8);
-      const fprt::BufView yv = fprt::make_buf(((SFX && c2.sfx) ? Ysg : Yg) + (c2.ok ? rowsB(c2) : 0),
-                                              c2.ok ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u);
+      const bool live = c2.ok && !STATE;
+      const fprt::BufView yv = fprt::make_buf(((SFX && c2.sfx) ? Ysg : Yg) + (live ? rowsB(c2) : 0),
+                                              live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u);
       fprt::buf_store128(yv, yg_off, v0);
       fprt::buf_store128(yv, yg_off + 16, v1);
     };
@@ -304,7 +308,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       const int L = ck.L;
       const Chunk ck2 = chunk_after(ck1);
       feed_load(refill, ck2);
-      drain_y(ckp, s ^ 1);
+      if (!STATE) drain_y(ckp, s ^ 1);
       const uint16_t* xs = XS + s * CH * X_LD;
       const uint16_t* ws = WS + s * CH * X_LD;
       const uint16_t* zt = ZT + s * BV * T_LD;
@@ -320,6 +324,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       }
 
       fprt::prof_stamp(it, 0);
+      if (STATE) {   // feed Z for the state waves, nothing else
+        feed_store_z(ready, s ^ 1);
+        fprt::block_sync();
+        ckp = ck;
+        ck = ck1;
+        ck1 = ck2;
+        return ck.ok;
+      }
       if (dbg & 2) {
         fprt::block_sync();
         ckp = ck;
@@ -609,7 +621,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   };
   auto store_rowmajor = [&](const ChunkRegs& cr, int s) {
     uint16_t* ws = WS + s * CH * X_LD;
-    if (ws_writer) {
+    if (ws_writer && !STATE) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) st128(ws + ws_off + r * X_LD, cr.w[r]);
     }
@@ -745,7 +757,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         }
       }
       if (BLOCKS && inj) tile_accumulate(t_inj, s ^ 1, true);
-      write_rt(s ^ 1);
+      if (!STATE) write_rt(s ^ 1);
     }
     fprt::prof_stamp(it, 4);
     fprt::block_sync();

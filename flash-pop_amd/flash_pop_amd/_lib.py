@@ -3,19 +3,22 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_void_p, POINTER, c_double
+from ctypes import c_char_p, c_int, c_size_t, c_void_p, POINTER, c_double
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libflashpop_hip.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
-_P, _I = c_void_p, c_int
+_P, _I, _Z = c_void_p, c_int, c_size_t
 _D = POINTER(c_double)
 
 # name -> argument types, in the order of include/flashpop_hip.h
 SIGNATURES = {
     "fp_retention_fwd": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P],
     "fp_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "fp_retention_workspace_bytes": [_I, _I, _I, _I, _I],
+    "fp_retention_fwd_split": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
+    "fp_retention_bwd_split": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
     "fp_pop_retention_fwd": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "fp_pop_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "fp_pop_fused_fwd": [_P] * 7 + [_D] + [_P] * 3 + [_I] * 7 + [_P],
@@ -33,7 +36,7 @@ def bind(path: str) -> ctypes.CDLL:
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
         fn.argtypes = argtypes
-        fn.restype = c_char_p if name == "fp_last_error" else c_int
+        fn.restype = {"fp_last_error": c_char_p, "fp_retention_workspace_bytes": c_size_t}.get(name, c_int)
     return lib
 
 

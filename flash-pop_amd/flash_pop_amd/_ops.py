@@ -35,14 +35,28 @@ def prepare(q, k, v, s, head_decays):
     return q, k, v, s, (B, T, H, dk, dv)
 
 
+def _workspace(lib, shape, device):
+    """Scratch for the split-sequence entry points: long sequences with few (batch, head) streams
+    are cut into segments so that the whole device works on them.  None when the library would not
+    cut this shape.  The tensor comes from torch's stream-ordered allocator, so handing it back
+    right after the call is safe."""
+    nbytes = lib.fp_retention_workspace_bytes(*shape)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
 def retention_fwd(q, k, v, s, decays, shape):
     lib = _lib.load()
     B, T, H, dk, dv = shape
     o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
     s_out = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
-        rc = lib.fp_retention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o), _ptr(s_out),
-                                  B, T, H, dk, dv, _stream())
+        ws = _workspace(lib, shape, q.device)
+        if ws is None:
+            rc = lib.fp_retention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
+                                      _ptr(s_out), B, T, H, dk, dv, _stream())
+        else:
+            rc = lib.fp_retention_fwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
+                                            _ptr(s_out), B, T, H, dk, dv, _ptr(ws), ws.numel(), _stream())
     _lib.check(lib, rc)
     return o, s_out
 
@@ -69,7 +83,12 @@ def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size,
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     d_s0 = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device) if want_ds0 else None
     with torch.cuda.device(q.device):
-        if block_size is None:
+        ws = _workspace(lib, shape, q.device) if block_size is None else None
+        if ws is not None:
+            rc = lib.fp_retention_bwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
+                                            _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
+                                            _ptr(ws), ws.numel(), _stream())
+        elif block_size is None:
             rc = lib.fp_retention_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                       _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
                                       _stream())

@@ -21,6 +21,8 @@
 #ifndef FLASHPOP_HIP_H
 #define FLASHPOP_HIP_H
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -49,6 +51,26 @@ int fp_retention_fwd(const void* q, const void* k, const void* v, const void* s0
 int fp_retention_bwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
                      const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B, int T,
                      int H, int dk, int dv, void* stream);
+
+/* Long sequences with few (batch, head) streams: one workgroup walks one stream, so B * H *
+ * min(dk, dv) / 64 workgroups is all a call has, and a 256-CU device idles when that is small.
+ * The _split variants cut every sequence into segments that run as separate sequences (a
+ * state-only pass and a scan give each segment its starting state first); they need scratch
+ * memory from the caller.  Same arguments, results and error behaviour as fp_retention_fwd /
+ * fp_retention_bwd otherwise; segment states pass through bf16.  No counterpart in the
+ * reference, whose kernels also walk a sequence serially (fused_chunk_fwd.py:95-187).
+ *   fp_retention_workspace_bytes  scratch bytes the two calls need for this shape on the current
+ *                                 device; 0 means they would not cut (and accept workspace = NULL)
+ *   workspace                     device memory, 16-byte aligned, at least that many bytes; its
+ *                                 contents are undefined afterwards, and two calls that share it
+ *                                 must be ordered by their stream */
+size_t fp_retention_workspace_bytes(int B, int T, int H, int dk, int dv);
+int fp_retention_fwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                           void* o, void* s_out, int B, int T, int H, int dk, int dv, void* workspace,
+                           size_t workspace_bytes, void* stream);
+int fp_retention_bwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                           const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B,
+                           int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Replaces the kernel call in FlashPOPRetention.forward
  * (flash_pop/pop_retention/__init__.py:14-31).

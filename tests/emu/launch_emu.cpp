@@ -3,6 +3,7 @@
 #include "device_rt.h"
 #include "retention_pass.h"
 #include "retention_pass_ws.h"
+#include "segment_scan.h"
 
 #include <thread>
 #include <vector>
@@ -61,6 +62,10 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
   if (a.slots <= 0) a.slots = (ws && !blocks && !suffix && a.B > 2) ? 2 : a.B;
   if (a.slots > a.B) a.slots = a.B;
   const bool multi = a.slots < a.B;
+  if (a.state_only && (!ws || blocks || suffix || !a.Rout)) {
+    *err = "state-only walk: needs dA of 64 or 128, a final-state buffer, no block states and no suffixes";
+    return 1;
+  }
   if (multi && (!ws || blocks || suffix)) {
     *err = "several batch entries per workgroup need the plain wave-specialised kernel";
     return 1;
@@ -70,15 +75,40 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
     case 64:
       if (suffix) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_SUFFIX>(a, l); });
       if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_BLOCKS>(a, l); });
+      if (a.state_only) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_STATE>(a, l); });
       if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_MULTI>(a, l); });
       return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_PLAIN>(a, l); });
     case 128:
       if (suffix) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_SUFFIX>(a, l); });
       if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_BLOCKS>(a, l); });
+      if (a.state_only) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_STATE>(a, l); });
       if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_MULTI>(a, l); });
       return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_PLAIN>(a, l); });
     case 256:
       return run_grid(fpk::NTHREADS, nwg, fpk::lds_bytes(256), [&](char* l) { fpk::retention_pass<256>(a, l); });
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
+}
+
+// Pretends the chip has 8 compute units, so that small test shapes take the paths that large
+// ones take on a real device (several sequences per workgroup, split sequences).
+int fpk_compute_units() { return 8; }
+
+int fpk_launch_scan(const fpk::ScanArgs& a, void* /*stream*/, const char** err) {
+  if (a.M % fpk::SCAN_VEC != 0 || a.B < 1 || a.S < 1 || a.H < 1 || !a.U || !a.init) {
+    *err = "segment scan: bad arguments";
+    return 1;
+  }
+  const long long items = (long long)a.B * a.H * (a.M / fpk::SCAN_VEC);
+  const int blocks = (int)((items + fpk::SCAN_THREADS - 1) / fpk::SCAN_THREADS);
+  // no barriers inside: the lanes can run one after another on this thread
+  for (int blk = 0; blk < blocks; ++blk) {
+    for (int t = 0; t < fpk::SCAN_THREADS; ++t) {
+      fprt::g_lane.tid = t;
+      fprt::g_lane.block = blk;
+      fprt::g_lane.grid = blocks;
+      fpk::segment_scan(a);
+    }
+  }
+  return 0;
 }

@@ -213,3 +213,30 @@ def raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot, stream=None, want_ds
                                      _p(cot[0]), _p(cot[1]), _p(cot[2]), *[_p(t) for t in outs], _p(ds0),
                                      B, T, H, dk, dv, block, Ls, stream))
     return outs + [ds0]
+
+
+def raw_split_fwd(lib, q, k, v, s, decays, stream=None):
+    """fp_retention_fwd_split with a workspace of exactly the size the library asks for.
+    Returns (o, s_out, workspace bytes)."""
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    nbytes = lib.fp_retention_workspace_bytes(B, T, H, dk, dv)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+    o = torch.full((B, T, H, dv), float("nan"), dtype=BF16, device=q.device)
+    S = torch.full((B, H, dk, dv), float("nan"), dtype=BF16, device=q.device)
+    _check(lib, lib.fp_retention_fwd_split(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o), _p(S), B, T, H, dk, dv,
+                                           _p(ws) if nbytes else None, nbytes, stream))
+    return o, S, nbytes
+
+
+def raw_split_bwd(lib, q, k, v, s, decays, d_o, d_s, stream=None):
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    nbytes = lib.fp_retention_workspace_bytes(B, T, H, dk, dv)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+    nan = lambda *shape: torch.full(shape, float("nan"), dtype=BF16, device=q.device)
+    dq, dk_, dv_, ds0 = nan(*q.shape), nan(*k.shape), nan(*v.shape), nan(B, H, dk, dv)
+    _check(lib, lib.fp_retention_bwd_split(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(d_o), _p(d_s), _p(dq), _p(dk_),
+                                           _p(dv_), _p(ds0), B, T, H, dk, dv, _p(ws) if nbytes else None, nbytes,
+                                           stream))
+    return dq, dk_, dv_, ds0

@@ -86,6 +86,22 @@ def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std):
     _check_all([(n, g, r) for n, g, r in zip(FUSED_NAMES, grads, g_ref)])
 
 
+@pytest.mark.parametrize("B,T,H,dk,dv,state_std,segments", [
+    (1, 512, 1, 64, 64, 0.5, 2),       # the harness pretends to have 8 compute units: 1 stream -> 2 segments of 4 chunks
+    (1, 1024, 1, 64, 128, None, 4),    # dk != dv, no initial state, 4 segments
+    (1, 256, 1, 64, 64, 0.5, 1),       # too short to cut: same path as the plain entry point
+])
+def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
+    decays = (0.97,) * H
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T, state_std=state_std)
+    d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=T + 1)
+    o, S, nbytes = hp.raw_split_fwd(emu_lib, q, k, v, s, decays)
+    assert nbytes == (2 * 2 * B * segments * H * dk * dv if segments > 1 else 0)
+    dq, dk_, dv_, ds0 = hp.raw_split_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
+    o_ref, S_ref, (gq, gk, gv, gs) = hp.oracle_plain(q, k, v, s, decays, d_o, d_s)
+    _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
+
+
 def test_optional_outputs_and_determinism(emu_lib):
     decays = oracle.head_decays(2)
     q, k, v, s = hp.make_inputs(1, 90, 2, 64, 64, seed=3, state_std=0.5)

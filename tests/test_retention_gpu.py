@@ -161,3 +161,39 @@ def test_recurrent_decode_matches_chunkwise():
         outs.append(o_t)
     hp.assert_close(torch.cat(outs, 1), o.float(), "decode o", rms_bar=2e-2)
     hp.assert_close(state, S.float(), "decode S", rms_bar=2e-2)
+
+
+def test_split_entry_points_long_sequence_few_streams():
+    """fp_retention_*_split on a shape the library cuts into segments (4 streams on a 256-CU device):
+    against the oracle, against the unsplit entry points, and the workspace argument checks."""
+    from flash_pop_amd import _lib
+    lib = _lib.load()
+    B, T, H, dk, dv = 1, 8192, 2, 128, 128
+    _say(f"[split] B{B} T{T} H{H} dk{dk} dv{dv}")
+    decays = oracle.head_decays(H, (5, 9))
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=77, state_std=0.05, device=DEV)
+    d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=78, device=DEV)
+    o, S, nbytes = hp.raw_split_fwd(lib, q, k, v, s, decays)
+    assert nbytes > 0 and nbytes % (2 * 2 * B * H * dk * dv) == 0, nbytes
+    grads = hp.raw_split_bwd(lib, q, k, v, s, decays, d_o, d_s)
+    o1, S1 = hp.raw_fwd(lib, q, k, v, s, decays)
+    grads1 = hp.raw_bwd(lib, q, k, v, s, decays, d_o, d_s)
+    torch.cuda.synchronize()
+    o_ref, S_ref, g_ref = hp.oracle_plain(q, k, v, s, decays, d_o, d_s)
+    names = ("dq", "dk", "dv", "ds0")
+    hp.assert_close(o, o_ref, "o", head_dim=2)
+    hp.assert_close(S, S_ref, "S", head_dim=1)
+    for n, g, r in zip(names, grads, g_ref):
+        hp.assert_close(g, r, n, head_dim=1 if n == "ds0" else 2)
+    # the two routes differ only by the bf16 rounding of the segment states
+    hp.assert_close(o, o1.float(), "o vs unsplit", head_dim=2)
+    for n, g, g1 in zip(names, grads, grads1):
+        hp.assert_close(g, g1.float(), f"{n} vs unsplit", head_dim=1 if n == "ds0" else 2)
+    # workspace checks happen before any launch
+    p, dec = hp._p, hp._dec(decays)
+    small = torch.empty(nbytes - 16, dtype=torch.uint8, device=DEV)
+    assert lib.fp_retention_fwd_split(p(q), p(k), p(v), p(s), dec, p(o), p(S), B, T, H, dk, dv, p(small), nbytes - 16, None) == -2
+    assert b"workspace" in lib.fp_last_error()
+    assert lib.fp_retention_fwd_split(p(q), p(k), p(v), p(s), dec, p(o), p(S), B, T, H, dk, dv, None, 0, None) == -1
+    # a shape that fills the device is not cut and needs no workspace
+    assert lib.fp_retention_workspace_bytes(8, 4096, 16, 128, 128) == 0
