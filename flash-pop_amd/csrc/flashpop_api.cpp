@@ -457,8 +457,24 @@ int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0
                         dk_, dv_, dq_sfx, dk_sfx, dv_sfx, d_s0, block_size, stream);
 }
 
+int fp_retention_decode_step(const void* q, const void* k, const void* v, const void* s_in, const double* head_decays,
+                             void* o, void* s_out, int B, int H, int dk, int dv, void* stream) {
+  const Shape s{B, 1, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (!q || !k || !v || !o || !s_out) return fail(FP_ERR_NULL_POINTER, "q, k, v, o and s_out must not be NULL");
+  fpk::DecodeArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.q = in(q); a.k = in(k); a.v = in(v); a.s_in = in(s_in); a.s_out = out(s_out); a.o = out(o);
+  a.B = B; a.H = H; a.dk = dk; a.dv = dv;
+  a.scale = 1.0f / std::sqrt((float)dk);
+  for (int h = 0; h < H; ++h) a.gamma[h] = (float)head_decays[h];
+  const char* msg = "";
+  if (fpk_launch_decode(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "decode step: %s", msg);
+  return FP_OK;
+}
+
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1002; }
+int fp_version(void) { return 1003; }
 
 }  // extern "C"

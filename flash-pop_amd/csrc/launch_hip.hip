@@ -3,6 +3,7 @@
 #include "retention_pass.h"
 #include "retention_pass_ws.h"
 #include "segment_scan.h"
+#include "decode_step.h"
 
 namespace {
 
@@ -22,6 +23,11 @@ __global__ __launch_bounds__(fpk::NTHREADS) void retention_pass_kernel(const fpk
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
   fpk::segment_scan(args);
+}
+
+__global__ __launch_bounds__(fpk::DECODE_THREADS) void decode_step_kernel(const fpk::DecodeArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::decode_step(args, lds);
 }
 
 template <typename Kernel>
@@ -146,6 +152,22 @@ int fpk_launch_scan(const fpk::ScanArgs& a, void* stream, const char** err) {
   }
   hipLaunchKernelGGL(segment_scan_kernel, dim3((unsigned)blocks), dim3(fpk::SCAN_THREADS), 0,
                      static_cast<hipStream_t>(stream), a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    *err = hipGetErrorString(e);
+    return 1;
+  }
+  return 0;
+}
+
+int fpk_launch_decode(const fpk::DecodeArgs& a, void* stream, const char** err) {
+  if (a.B < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || a.dk < 1 || a.dv < 8 || a.dv % 8 != 0 ||
+      fpk::DECODE_THREADS % (a.dv / 8) != 0 || a.dv > fpk::DECODE_THREADS || !a.q || !a.k || !a.v || !a.s_out || !a.o) {
+    *err = "decode step: bad arguments";
+    return 1;
+  }
+  hipLaunchKernelGGL(decode_step_kernel, dim3((unsigned)(a.B * a.H)), dim3(fpk::DECODE_THREADS),
+                     fpk::decode_lds_bytes(a.dv), static_cast<hipStream_t>(stream), a);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     *err = hipGetErrorString(e);

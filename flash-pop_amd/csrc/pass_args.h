@@ -75,6 +75,22 @@ struct ScanArgs {
   int B, S, H, M, Tseg, reverse;
   float log2g[MAX_HEADS];
 };
+// One recurrent (decode) step for every (batch, head):  S' = gamma S + (scale k)^T v,  o = q S'.
+// q, k [B,H,dk]; v, o [B,H,dv]; S [B,H,dk,dv]; all bf16, fp32 arithmetic.  s_out may be s_in.
+struct DecodeArgs {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  const uint16_t* s_in;   // nullable (zeros)
+  uint16_t* s_out;
+  uint16_t* o;
+  int B, H, dk, dv;
+  float scale;
+  float gamma[MAX_HEADS];
+};
+constexpr int DECODE_THREADS = 256;
+constexpr int decode_lds_bytes(int dv) { return (DECODE_THREADS / (dv / 8)) * dv * 4; }
+
 constexpr int SCAN_THREADS = 256;
 constexpr int SCAN_VEC = 8;   // elements per thread
 
@@ -89,3 +105,6 @@ int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);
 
 // Compute units of the current device (what the launcher sizes its grids against).
 int fpk_compute_units();
+
+// Launches the decode-step kernel.  Same conventions as fpk_launch_pass.
+int fpk_launch_decode(const fpk::DecodeArgs& args, void* stream, const char** err);

@@ -2,6 +2,7 @@
 from .fused_retention import fused_chunk_retention, FusedChunkRetention  # noqa: F401
 from .pop_retention import (  # noqa: F401
     flash_pop_retention, FlashPOPRetention, flash_pop_retention_with_suffixes, FlashPOPRetentionWithSuffixes)
+from .recurrent import retention_recurrent  # noqa: F401
 
-__all__ = ["fused_chunk_retention", "flash_pop_retention", "flash_pop_retention_with_suffixes",
+__all__ = ["retention_recurrent", "fused_chunk_retention", "flash_pop_retention", "flash_pop_retention_with_suffixes",
            "FusedChunkRetention", "FlashPOPRetention", "FlashPOPRetentionWithSuffixes"]

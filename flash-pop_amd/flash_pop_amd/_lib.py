@@ -23,6 +23,7 @@ SIGNATURES = {
     "fp_pop_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "fp_pop_fused_fwd": [_P] * 7 + [_D] + [_P] * 3 + [_I] * 7 + [_P],
     "fp_pop_fused_bwd": [_P] * 7 + [_D] + [_P] * 10 + [_I] * 7 + [_P],
+    "fp_retention_decode_step": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _P],
     "fp_last_error": [],
     "fp_version": [],
 }

@@ -147,3 +147,35 @@ def pop_fused_bwd(q, k, v, s, sfx, decays, block_size, shape, d_o, d_o_sfx, d_s_
                                   sfx[0].shape[1], _stream())
     _lib.check(lib, rc)
     return outs, d_s0
+
+
+def decode_step(q, k, v, s, decays, in_place=False):
+    """q, k [B,H,dk], v [B,H,dv], s [B,H,dk,dv] or None -> (o [B,H,dv], new state)."""
+    lib = _lib.load()
+    if q.dim() != 3 or k.shape != q.shape or v.dim() != 3 or v.shape[:2] != q.shape[:2]:
+        raise ValueError(f"expected q, k [B,H,dk] and v [B,H,dv]; got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    B, H, dk = q.shape
+    dv = v.shape[2]
+    assert len(decays) == H, f"got {len(decays)} head decays for {H} heads"
+    for name, t in (("q", q), ("k", k), ("v", v), ("s", s)):
+        if t is None:
+            continue
+        assert t.dtype == torch.bfloat16, f"{name}: only bfloat16 is supported, got {t.dtype}"
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}: flash_pop_amd runs on the GPU only")
+    if s is not None and tuple(s.shape) != (B, H, dk, dv):
+        raise ValueError(f"expected state [B,H,dk,dv] = {(B, H, dk, dv)}, got {tuple(s.shape)}")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    if in_place:
+        if s is None or not s.is_contiguous():
+            raise ValueError("an in-place step needs a contiguous state tensor")
+        s_out = s
+    else:
+        s = None if s is None else s.contiguous()
+        s_out = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device)
+    o = torch.empty((B, H, dv), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.fp_retention_decode_step(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
+                                          _ptr(s_out), B, H, dk, dv, _stream())
+    _lib.check(lib, rc)
+    return o, s_out

@@ -114,6 +114,14 @@ int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0
                      const void* d_s_out, void* dq, void* dk_, void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx,
                      void* d_s0, int B, int T, int H, int dk, int dv, int block_size, int sfx_len, void* stream);
 
+/* One recurrent (decode) step for all batch entries and heads in one launch; replaces the
+ * einsums of retention_recurrent (flash_pop/retnet.py:79-101):
+ *   S' = gamma_h S + (k / sqrt(dk))^T v,   o = q S'
+ *   q, k [B,H,dk]; v, o [B,H,dv]; s_in (may be NULL: zeros), s_out [B,H,dk,dv]; s_out may be s_in
+ * The state is read once and written once; arithmetic in fp32, storage bf16. */
+int fp_retention_decode_step(const void* q, const void* k, const void* v, const void* s_in, const double* head_decays,
+                             void* o, void* s_out, int B, int H, int dk, int dv, void* stream);
+
 /* Message for the last nonzero return on this thread ("" if none). */
 const char* fp_last_error(void);
 

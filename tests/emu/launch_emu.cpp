@@ -4,6 +4,7 @@
 #include "retention_pass.h"
 #include "retention_pass_ws.h"
 #include "segment_scan.h"
+#include "decode_step.h"
 
 #include <thread>
 #include <vector>
@@ -111,4 +112,13 @@ int fpk_launch_scan(const fpk::ScanArgs& a, void* /*stream*/, const char** err) 
     }
   }
   return 0;
+}
+
+int fpk_launch_decode(const fpk::DecodeArgs& a, void* /*stream*/, const char** err) {
+  if (a.B < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || a.dk < 1 || a.dv < 8 || a.dv % 8 != 0 ||
+      fpk::DECODE_THREADS % (a.dv / 8) != 0 || a.dv > fpk::DECODE_THREADS || !a.q || !a.k || !a.v || !a.s_out || !a.o) {
+    *err = "decode step: bad arguments";
+    return 1;
+  }
+  return run_grid(fpk::DECODE_THREADS, a.B * a.H, fpk::decode_lds_bytes(a.dv), [&](char* l) { fpk::decode_step(a, l); });
 }

@@ -240,3 +240,13 @@ def raw_split_bwd(lib, q, k, v, s, decays, d_o, d_s, stream=None):
                                            _p(dv_), _p(ds0), B, T, H, dk, dv, _p(ws) if nbytes else None, nbytes,
                                            stream))
     return dq, dk_, dv_, ds0
+
+
+def raw_decode_step(lib, q, k, v, s, decays, stream=None, in_place=False):
+    B, H, dk = q.shape
+    dv = v.shape[2]
+    o = torch.full((B, H, dv), float("nan"), dtype=BF16, device=q.device)
+    s_out = s if in_place else torch.full((B, H, dk, dv), float("nan"), dtype=BF16, device=q.device)
+    _check(lib, lib.fp_retention_decode_step(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o), _p(s_out), B, H, dk, dv,
+                                             stream))
+    return o, s_out

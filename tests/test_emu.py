@@ -102,6 +102,22 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
 
 
+@pytest.mark.parametrize("B,H,dk,dv", [(2, 3, 64, 128), (1, 2, 128, 64), (1, 1, 256, 256)])
+def test_decode_step(emu_lib, B, H, dk, dv):
+    """Three chained steps (no state, fresh buffer, in place) against the oracle's recurrent step."""
+    decays = oracle.head_decays(H)
+    g = torch.Generator().manual_seed(dk + dv)
+    state, ref_state = None, None
+    for step in range(3):
+        q, k = (torch.randn(B, H, dk, generator=g).to(hp.BF16) for _ in range(2))
+        v = torch.randn(B, H, dv, generator=g).to(hp.BF16)
+        o, state = hp.raw_decode_step(emu_lib, q, k, v, state, decays, in_place=step == 2)
+        o_ref, ref_state = oracle.recurrent_step(q.float(), k.float(), v.float(), ref_state, decays)
+        hp.assert_close(o, o_ref, f"o step {step}")
+        hp.assert_close(state, ref_state, f"state step {step}")
+        ref_state = state.float()    # follow the kernel's bf16 state, as a decode loop does
+
+
 def test_optional_outputs_and_determinism(emu_lib):
     decays = oracle.head_decays(2)
     q, k, v, s = hp.make_inputs(1, 90, 2, 64, 64, seed=3, state_std=0.5)

@@ -163,6 +163,44 @@ def test_recurrent_decode_matches_chunkwise():
     hp.assert_close(state, S.float(), "decode S", rms_bar=2e-2)
 
 
+def test_decode_step_kernel_256_steps():
+    """retention_recurrent (one launch per step for all heads) over 256 steps, the state carried in
+    bf16 and updated in place as a decode loop does, against the oracle run over the whole sequence
+    (config-5 head dims: dk 64, dv 128, 12 heads)."""
+    from flash_pop_amd import retention_recurrent
+    B, T, H, dk, dv = 4, 256, 12, 64, 128
+    _say(f"[decode] B{B} T{T} H{H} dk{dk} dv{dv}")
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=91, state_std=0.1)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    state = s.to(DEV).clone()
+    outs = []
+    for t in range(T):
+        o_t, state = retention_recurrent(qd[:, t], kd[:, t], vd[:, t], decays, state, in_place=True)
+        outs.append(o_t)
+    o = torch.stack(outs, dim=1)
+    # first step without a state, fresh output buffer
+    o0, s1 = retention_recurrent(qd[:, 0], kd[:, 0], vd[:, 0], decays, None)
+    torch.cuda.synchronize()
+    # step by step, with the state rounded to bf16 after every step as the kernel stores it
+    ref_state, ref_outs = s.float(), []
+    for t in range(T):
+        o_t, ref_state = oracle.recurrent_step(q[:, t].float(), k[:, t].float(), v[:, t].float(), ref_state, decays)
+        ref_state = ref_state.to(hp.BF16).float()
+        ref_outs.append(o_t)
+    hp.assert_close(o, torch.stack(ref_outs, dim=1), "o", head_dim=2)
+    hp.assert_close(state, ref_state, "final state", head_dim=1)
+    # against the exact sequence result the bf16 state adds a rounding error per step that the slowly
+    # decaying heads accumulate (about sqrt(T) * 2^-9 / sqrt(3)); the reference's decode loop carries
+    # its state in bf16 in the same way
+    o_ref, S_ref = hp.oracle_plain(q, k, v, s, decays)
+    assert oracle.rms_error_ratio(o.float().cpu(), o_ref) < 3e-2
+    assert oracle.rms_error_ratio(state.float().cpu(), S_ref) < 3e-2
+    o0_ref, s1_ref = oracle.recurrent_step(q[:, 0].float(), k[:, 0].float(), v[:, 0].float(), None, decays)
+    hp.assert_close(o0, o0_ref, "o, no state")
+    hp.assert_close(s1, s1_ref, "state, no state")
+
+
 def test_split_entry_points_long_sequence_few_streams():
     """fp_retention_*_split on a shape the library cuts into segments (4 streams on a 256-CU device):
     against the oracle, against the unsplit entry points, and the workspace argument checks."""
