@@ -6,7 +6,7 @@ resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic F
 (dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the pass kernel measured
 with events on the launch stream, and the CPU oracle timed on the host cores beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop] [--no-long]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop] [--no-long] [--no-model]
 """
 import argparse
 import json
@@ -203,7 +203,62 @@ def gpu_leg(args):
             "segments_per_sequence": _lib.load().fp_retention_workspace_bytes(B3, T3, H3, dk3, dv3)
             // (4 * B3 * H3 * dk3 * dv3),
         }
+    if not args.no_model:
+        out["model"] = model_leg(args, dev)
     return out
+
+
+def model_leg(args, dev):
+    """Config 5: a random-init 12-layer POP-RetNet decoder (tests/model_harness.py) on the HIP ops:
+    one POP training step (fwd+bwd, B=8, T=2048 in 64-token blocks with 16-token suffixes), then
+    256 recurrent decode steps from the states it leaves."""
+    import torch
+    import model_harness as mh
+
+    cfg = mh.HarnessConfig()
+    B, T, decode_steps = 8, 2048, 256
+    backend = mh.HipBackend()
+    model = mh.build(cfg, seed=0, device=dev)
+    batch = mh.synthetic_batch(cfg, B, T, seed=1, device=dev)
+
+    def train_step():
+        model.zero_grad(set_to_none=True)
+        loss, _, _, states = mh.pop_loss(model, backend, batch)
+        loss.backward()
+        return states
+
+    for _ in range(2):
+        train_step()
+    torch.cuda.synchronize()
+    n = max(3, args.steps // 10)
+    t0 = time.perf_counter()
+    for _ in range(n):
+        states = train_step()
+    torch.cuda.synchronize()
+    train_ms = (time.perf_counter() - t0) * 1e3 / n
+
+    states = [s.detach() for s in states]
+    token = batch[0][:, -1]
+    with torch.no_grad():
+        for i in range(8):
+            logits, states = model.recurrent(backend, token, states, T + i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(decode_steps):
+            logits, states = model.recurrent(backend, token, states, T + 8 + i)
+            token = logits.argmax(-1)
+        torch.cuda.synchronize()
+    decode_ms = (time.perf_counter() - t0) * 1e3 / decode_steps
+    tokens = B * T + B * (T // cfg.block + 1) * cfg.sfx_len
+    return {
+        "workload": "config 5: 12-layer POP-RetNet decoder d_model=768 H=12 dk=64 dv=128 FFN=3072 vocab=32000, "
+                    "bf16, B=8 T=2048, 64-token blocks, 16-token suffixes; eager torch around the HIP retention ops",
+        "train_step_ms": round(train_ms, 2),
+        "train_tokens_per_s": round(tokens / (train_ms * 1e-3), 1),
+        "decode_steps": decode_steps,
+        "decode_ms_per_step": round(decode_ms, 3),
+        "decode_tokens_per_s": round(B / (decode_ms * 1e-3), 1),
+    }
 
 
 def cpu_leg(sample_batch=1, reps=2):
@@ -246,6 +301,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
     ap.add_argument("--no-long", action="store_true", help="skip the long-context (config 3) timing")
+    ap.add_argument("--no-model", action="store_true", help="skip the model-level (config 5) timing")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy (scales the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()

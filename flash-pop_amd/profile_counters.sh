@@ -8,7 +8,7 @@ R=$(cd "$(dirname "$0")/.." && pwd)
 O=$R/gpurun_out/profile
 mkdir -p "$O"
 cd /tmp && export TMPDIR=/tmp
-BENCH="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu"
+BENCH="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu --no-long --no-model"
 COPY="python3 $R/bench.py --copy-calibration"
 run() { name=$1; shift; timeout -s KILL 120 rocprofv3 "$@" --output-format csv -d "$O/$name" -o r -- $CMD > "$O/$name.log" 2>&1; }
 CMD=$BENCH run trace --kernel-trace --stats

@@ -1,0 +1,243 @@
+"""A minimal POP-RetNet decoder around the retention ops, for model-level parity tests and the
+model leg of the benchmark.  Test infrastructure: plain torch modules, written for this harness.
+
+It follows the structure of the reference's model (flash_pop/retnet.py:105-366 multi-scale
+retention, :370-512 decoder layer, flash_pop/pop_retnet.py:82-171 POP layer step,
+flash_pop/xpos_emb.py rotary embedding): pre-LayerNorm in fp32, q/k rotated by position * theta,
+retention, GroupNorm over each head's outputs (fp32, no affine, eps 1e-6), swish gate, output
+projection, swish FFN.  Unlike the reference, d_model need not equal H * dv: v and the gate are
+projected d_model -> H * dv and the output H * dv -> d_model, which reduces to the reference's
+layer when the two are equal.
+
+The retention itself comes from a backend object, so that the same seeded model can run on the
+HIP ops and on the CPU oracle's formulas (evaluated on whatever device the tensors are on).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+
+@dataclass
+class HarnessConfig:
+    vocab: int = 32000
+    d_model: int = 768
+    layers: int = 12
+    heads: int = 12
+    dk: int = 64
+    dv: int = 128
+    ffn: int = 3072
+    block: int = 64          # context tokens per observation block
+    sfx_len: int = 16        # prediction tokens per POP suffix
+    dtype: torch.dtype = torch.bfloat16
+
+
+def head_decays(heads: int) -> tuple:
+    return tuple(1.0 - 2.0 ** (-5.0 - h) for h in range(heads))       # flash_pop/retnet.py:70-76
+
+
+class HipBackend:
+    """The ops of flash_pop_amd."""
+    name = "hip"
+
+    def plain(self, q, k, v, s, decays):
+        from flash_pop_amd import fused_chunk_retention
+        return fused_chunk_retention(q, k, v, s, decays)
+
+    def pop(self, q, k, v, s, decays, block, q_s, k_s, v_s):
+        from flash_pop_amd import flash_pop_retention_with_suffixes
+        return flash_pop_retention_with_suffixes(q, k, v, s, decays, block, q_s, k_s, v_s)
+
+    def step(self, q, k, v, s, decays):
+        from flash_pop_amd import retention_recurrent
+        return retention_recurrent(q, k, v, decays, s)
+
+
+class OracleBackend:
+    """The oracle's formulas in fp32 on the bf16 inputs, results rounded to bf16 like the ops' outputs."""
+    name = "oracle"
+
+    def plain(self, q, k, v, s, decays):
+        import oracle
+        o, S = oracle.chunkwise_retention(q.float(), k.float(), v.float(), None if s is None else s.float(), decays, 64)
+        return o.to(q.dtype), S.to(q.dtype)
+
+    def pop(self, q, k, v, s, decays, block, q_s, k_s, v_s):
+        import oracle
+        f = lambda t: None if t is None else t.float()
+        o, o_s, last = oracle.pop_fused_retention(f(q), f(k), f(v), f(s), f(q_s), f(k_s), f(v_s), decays, block)
+        return o.to(q.dtype), o_s.to(q.dtype), last.to(q.dtype)
+
+    def step(self, q, k, v, s, decays):
+        import oracle
+        o, S = oracle.recurrent_step(q.float(), k.float(), v.float(), None if s is None else s.float(), decays)
+        return o.to(q.dtype), S.to(q.dtype)
+
+
+def rotate(x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """Pairs (x[2i], x[2i+1]) rotated by position * theta_i, theta_i = 10000^(-i / (d/2 - 1))
+    (flash_pop/xpos_emb.py:24-40).  x [..., n, h, d]; positions broadcastable to [..., n]."""
+    d = x.shape[-1]
+    theta = 1.0 / (10000.0 ** torch.linspace(0, 1, d // 2, device=x.device))
+    ang = positions[..., None, None].float() * theta                     # [..., n, 1, d/2]
+    sin, cos = torch.sin(ang), torch.cos(ang)
+    xf = x.float()
+    even, odd = xf[..., 0::2], xf[..., 1::2]
+    out = torch.stack((even * cos - odd * sin, odd * cos + even * sin), dim=-1).flatten(-2)
+    return out.to(x.dtype)
+
+
+class Retention(nn.Module):
+    def __init__(self, cfg: HarnessConfig):
+        super().__init__()
+        self.cfg = cfg
+        D, H, dk, dv = cfg.d_model, cfg.heads, cfg.dk, cfg.dv
+        self.q_proj = nn.Linear(D, H * dk)
+        self.k_proj = nn.Linear(D, H * dk)
+        self.v_proj = nn.Linear(D, H * dv)
+        self.g_proj = nn.Linear(D, H * dv)
+        self.out_proj = nn.Linear(H * dv, D)
+        for lin in (self.q_proj, self.k_proj, self.v_proj, self.g_proj, self.out_proj):
+            nn.init.xavier_normal_(lin.weight)
+            nn.init.zeros_(lin.bias)
+        self.decays = head_decays(H)
+
+    def qkv(self, x, positions):
+        H, dk, dv = self.cfg.heads, self.cfg.dk, self.cfg.dv
+        q = rotate(self.q_proj(x).unflatten(-1, (H, dk)), positions)
+        k = rotate(self.k_proj(x).unflatten(-1, (H, dk)), positions)
+        v = self.v_proj(x).unflatten(-1, (H, dv))
+        return q, k, v
+
+    def finish(self, x, retention):
+        """GroupNorm per head in fp32, gate, output projection.  retention [..., H, dv]."""
+        H = self.cfg.heads
+        r = retention.float()
+        r = (r - r.mean(-1, keepdim=True)) * torch.rsqrt(r.var(-1, unbiased=False, keepdim=True) + 1e-6)
+        r = r.flatten(-2).to(x.dtype)
+        return self.out_proj(r * F.silu(self.g_proj(x)))
+
+
+class Layer(nn.Module):
+    def __init__(self, cfg: HarnessConfig):
+        super().__init__()
+        self.cfg = cfg
+        self.norm1 = nn.LayerNorm(cfg.d_model, eps=1e-6)
+        self.norm2 = nn.LayerNorm(cfg.d_model, eps=1e-6)
+        self.retention = Retention(cfg)
+        self.linear1 = nn.Linear(cfg.d_model, cfg.ffn)
+        self.linear2 = nn.Linear(cfg.ffn, cfg.d_model)
+        for lin in (self.linear1, self.linear2):
+            nn.init.xavier_normal_(lin.weight)
+            nn.init.zeros_(lin.bias)
+
+    def _norm(self, norm, x):
+        return F.layer_norm(x.float(), (self.cfg.d_model,), norm.weight.float(), norm.bias.float(), norm.eps).to(x.dtype)
+
+    def _ffn(self, x):
+        return x + self.linear2(F.silu(self.linear1(self._norm(self.norm2, x))))
+
+    def pop_forward(self, backend, x, sfx, start, state):
+        """x [B,T,D], sfx [B*(N+1), Ls, D]: the layer step of flash_pop/pop_retnet.py:82-150, with
+        both retentions handed to the backend in one call.  Returns (x, sfx, last state)."""
+        r, cfg = self.retention, self.cfg
+        B, T = x.shape[:2]
+        n1 = sfx.shape[0] // B
+        xn, sn = self._norm(self.norm1, x), self._norm(self.norm1, sfx)
+        pos = start + torch.arange(T, device=x.device)
+        sfx_start = (start + torch.arange(n1, device=x.device) * cfg.block).repeat(B)       # pop_retnet.py:175-179
+        spos = sfx_start[:, None] + torch.arange(sfx.shape[1], device=x.device)[None]
+        q, k, v = r.qkv(xn, pos)
+        qs, ks, vs = r.qkv(sn, spos)
+        o, o_s, last = backend.pop(q, k, v, state, r.decays, cfg.block, qs, ks, vs)
+        x = self._ffn(x + r.finish(xn, o))
+        sfx = self._ffn(sfx + r.finish(sn, o_s))
+        return x, sfx, last
+
+    def chunkwise(self, backend, x, start, state):
+        r = self.retention
+        xn = self._norm(self.norm1, x)
+        q, k, v = r.qkv(xn, start + torch.arange(x.shape[1], device=x.device))
+        o, state = backend.plain(q, k, v, state, r.decays)
+        return self._ffn(x + r.finish(xn, o)), state
+
+    def recurrent(self, backend, x, index, state):
+        """x [B, D], one token (flash_pop/retnet.py:325-366, 493-512)."""
+        r = self.retention
+        xn = self._norm(self.norm1, x)
+        q, k, v = r.qkv(xn[:, None], torch.full((1,), index, device=x.device))
+        o, state = backend.step(q[:, 0], k[:, 0], v[:, 0], state, r.decays)
+        return self._ffn(x + r.finish(xn, o)), state
+
+
+class PopRetNetLM(nn.Module):
+    def __init__(self, cfg: HarnessConfig):
+        super().__init__()
+        self.cfg = cfg
+        self.embed = nn.Embedding(cfg.vocab, cfg.d_model)
+        self.layers = nn.ModuleList(Layer(cfg) for _ in range(cfg.layers))
+        self.norm = nn.LayerNorm(cfg.d_model, eps=1e-6)
+        self.head = nn.Linear(cfg.d_model, cfg.vocab, bias=False)
+        nn.init.normal_(self.embed.weight, std=cfg.d_model ** -0.5)
+        nn.init.normal_(self.head.weight, std=cfg.d_model ** -0.5)
+
+    def _logits(self, x):
+        x = F.layer_norm(x.float(), (self.cfg.d_model,), self.norm.weight.float(), self.norm.bias.float(), self.norm.eps)
+        return self.head(x.to(self.cfg.dtype))
+
+    def pop_forward(self, backend, tokens, sfx_tokens, states: Optional[List] = None, start: int = 0):
+        """tokens [B,T] (T a multiple of the block), sfx_tokens [B*(T/block + 1), Ls].
+        Returns (context logits, suffix logits, per-layer last states)."""
+        x, sfx = self.embed(tokens), self.embed(sfx_tokens)
+        states = states if states is not None else [None] * len(self.layers)
+        new_states = []
+        for layer, st in zip(self.layers, states):
+            x, sfx, last = layer.pop_forward(backend, x, sfx, start, st)
+            new_states.append(last)
+        return self._logits(x), self._logits(sfx), new_states
+
+    def chunkwise(self, backend, tokens, states: Optional[List] = None, start: int = 0):
+        x = self.embed(tokens)
+        states = states if states is not None else [None] * len(self.layers)
+        new_states = []
+        for layer, st in zip(self.layers, states):
+            x, st = layer.chunkwise(backend, x, start, st)
+            new_states.append(st)
+        return self._logits(x), new_states
+
+    @torch.no_grad()
+    def recurrent(self, backend, token, states: List, index: int):
+        """One decode step: token [B] -> (logits [B, vocab], new states)."""
+        x = self.embed(token)
+        new_states = []
+        for layer, st in zip(self.layers, states):
+            x, st = layer.recurrent(backend, x, index, st)
+            new_states.append(st)
+        return self._logits(x), new_states
+
+
+def build(cfg: HarnessConfig, seed: int, device) -> PopRetNetLM:
+    torch.manual_seed(seed)
+    model = PopRetNetLM(cfg)          # initialised on the CPU: the same weights whatever the device
+    return model.to(device=device, dtype=cfg.dtype)
+
+
+def synthetic_batch(cfg: HarnessConfig, B: int, T: int, seed: int, device):
+    """Uniform random token ids for the context, the suffixes and their next-token targets."""
+    g = torch.Generator().manual_seed(seed)
+    n1 = T // cfg.block + 1
+    draw = lambda *shape: torch.randint(0, cfg.vocab, shape, generator=g).to(device)
+    return draw(B, T), draw(B * n1, cfg.sfx_len), draw(B, T), draw(B * n1, cfg.sfx_len)
+
+
+def pop_loss(model: PopRetNetLM, backend, batch):
+    tokens, sfx_tokens, targets, sfx_targets = batch
+    logits, sfx_logits, states = model.pop_forward(backend, tokens, sfx_tokens)
+    loss = F.cross_entropy(logits.float().flatten(0, 1), targets.flatten()) + \
+        F.cross_entropy(sfx_logits.float().flatten(0, 1), sfx_targets.flatten())
+    return loss, logits, sfx_logits, states
