@@ -103,7 +103,7 @@ def gpu_leg(args):
         "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "retention_pass_ws_kernel<128, 0>",
+            "kernel": "retention_pass_ws_kernel<128, 0, 1>",
             "achieved": round(achieved_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -4,7 +4,7 @@
 // The whole state is read once and written once, which is all the HBM traffic the step has.
 #pragma once
 #include "pass_args.h"
-#include "retention_pass.h"   // ld/st and bf16 helpers
+#include "lds_access.h"
 
 namespace fpk {
 

@@ -1,24 +1,16 @@
 // gfx950 entry points of the pass kernels and the launcher the C-ABI layer calls.
 #include "device_rt.h"
-#include "retention_pass.h"
 #include "retention_pass_ws.h"
 #include "segment_scan.h"
 #include "decode_step.h"
 
 namespace {
 
-// dA = 64, 128: wave-specialised, 8 waves, double-buffered LDS.
-template <int DA, int MODE>
+// 8 waves, double-buffered LDS; NH = 2 covers dA = 256 in two visits per chunk.
+template <int DA, int MODE, int NH = 1>
 __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::retention_pass_ws<DA, MODE>(args, lds);
-}
-
-// dA = 256: 4 symmetric waves, single-buffered LDS (two stages of 256-wide tiles do not fit).
-template <int DA>
-__global__ __launch_bounds__(fpk::NTHREADS) void retention_pass_kernel(const fpk::PassArgs args) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::retention_pass<DA>(args, lds);
+  fpk::retention_pass_ws<DA, MODE, NH>(args, lds);
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -85,7 +77,7 @@ int fpk_compute_units() {
 
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  static thread_local int armed[11] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
+  static thread_local int armed[12] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
   fpk::PassArgs a = args;
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool ws = a.dA == 64 || a.dA == 128;
@@ -117,7 +109,7 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
     return 1;
   }
   if (multi && (!ws || blocks || suffix)) {
-    *err = "several batch entries per workgroup need the plain wave-specialised kernel";
+    *err = "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
     return 1;
   }
   switch (a.dA) {
@@ -133,8 +125,9 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
       if (a.state_only) return launch(retention_pass_ws_kernel<128, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[10], a, s, err);
       if (multi) return launch(retention_pass_ws_kernel<128, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[4], a, s, err);
       return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[5], a, s, err);
-    case 256:
-      return launch(retention_pass_kernel<256>, fpk::NTHREADS, fpk::lds_bytes(256), &armed[6], a, s, err);
+    case 256:   // two visits per chunk, 128 of the 256 contraction columns each
+      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[6], a, s, err);
+      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[11], a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }

@@ -21,7 +21,6 @@ namespace fpk {
 
 constexpr int CH = 64;          // tokens per chunk
 constexpr int BV = 64;          // columns of Z / Y / R owned by one workgroup
-constexpr int NTHREADS = 256;   // 4 wave64
 constexpr int MAX_HEADS = 128;
 
 struct PassArgs {
@@ -51,15 +50,6 @@ struct PassArgs {
   float s_intra, s_read, s_update;
   float log2g[MAX_HEADS];
 };
-
-// LDS bytes the pass kernel needs for a given dA.
-constexpr int lds_bytes(int dA) {
-  return 2 * (2 * CH * (dA + 8)      // X and W tiles, row-major
-              + dA * (CH + 4)        // weighted W, transposed
-              + BV * (CH + 4)        // Z, transposed
-              + BV * (dA + 8)        // bf16 copy of R, transposed
-              + CH * (BV + 8));      // Y staging
-}
 
 // Arguments of the segment scan that stitches a sequence cut into S segments back together.
 // U[b][s] is the state a segment contributes on its own (zero initial state); with g = gamma^Tseg

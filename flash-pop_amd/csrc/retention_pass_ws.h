@@ -1,4 +1,5 @@
-// Wave-specialised retention pass (see pass_args.h for the recurrence), dA = 64 or 128.
+// Wave-specialised retention pass (see pass_args.h for the recurrence): dA = 64 or 128 per visit,
+// dA = 256 in two visits per chunk (NH = 2 below).
 //
 // One workgroup of 8 wave64 owns one (batch, head) stream and one 64-column slice of
 // Z / Y / R.  Hardware places waves w and w + 4 on the same SIMD, so every SIMD runs one
@@ -26,7 +27,7 @@
 // and the vector work of one phase sits in the shadow of the next phase's MFMAs.
 #pragma once
 #include "pass_args.h"
-#include "retention_pass.h"   // ld/st helpers, acc_row
+#include "lds_access.h"
 
 namespace fpk {
 
@@ -39,6 +40,11 @@ constexpr int lds_bytes_ws(int dA) {
               + 2 * CH * (BV + 8)      // Y staging, two stages
               + 4 * 32 * (CH + 4));    // weighted W transposed, one 32-row slab per state wave
 }
+
+template <int H>
+struct Half {
+  static constexpr int value = H;
+};
 
 // two 8-byte LDS reads that form one MFMA operand: tokens 16 kt + 4 g + {0..3} and + 8
 FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
@@ -60,9 +66,16 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 //              the readout waves feed Z and do nothing else, X is not read and Y not written.
 enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WALK_STATE = 4 };
 
-template <int DA, int MODE>
+//
+// NH = 2 handles a contraction width of 2 DA (p.dA = 256 with DA = 128) with the LDS footprint of
+// DA: every chunk is visited twice, once per half of the columns of X and W (of the rows of R).
+// Scores and read-out are sums over the contraction index, so the readout waves simply keep
+// accumulating across the two visits and convert, multiply by Z and store only after the second;
+// the state waves carry one set of accumulators per half and update the half being visited.
+template <int DA, int MODE, int NH = 1>
 FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
+  static_assert(NH == 1 || (NH == 2 && (MODE == WALK_PLAIN || MODE == WALK_BLOCKS)), "two halves: plain and block walks only");
   constexpr bool STATE = MODE == WALK_STATE;
   constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI || STATE, SFX = MODE == WALK_SUFFIX;
   constexpr int X_LD = DA + 8;
@@ -130,8 +143,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     bool ok, first, last;   // exists / first item of its sequence / last item of its sequence
     bool sfx;               // a suffix (t0 is its block boundary) rather than a context chunk
     int n;                  // WALK_SUFFIX only: index of the suffix, or of the context chunk's block
+    int h;                  // NH = 2 only: which half of the contraction this visit covers
   };
-  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0};
+  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0, 0};
   auto first_chunk = [&](int b) {
     Chunk ck = {b, 0, 0, b < p.B, true, false, false, 0};
     if (ck.ok) {
@@ -149,6 +163,12 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   };
   auto chunk_after = [&](const Chunk& ck) {
     if (!ck.ok) return ck;
+    if (NH == 2 && ck.h == 0) {   // the same chunk again, other half
+      Chunk again = ck;
+      again.h = 1;
+      again.first = false;
+      return again;
+    }
     if (ck.last) return MULTI ? first_chunk(ck.b + p.slots) : no_chunk;
     Chunk n = {ck.b, 0, 0, true, false, false, false, 0};
     if (SFX) {
@@ -183,7 +203,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   auto first_row = [&](const Chunk& ck) {
     return (SFX && ck.sfx) ? ((size_t)ck.b * (p.nblk + 1) + ck.n) * p.Ls : (size_t)ck.b * T + ck.t0;
   };
-  auto rowsA = [&](const Chunk& ck) { return (first_row(ck) * p.H + h) * p.dA * 2; };
+  auto rowsA = [&](const Chunk& ck) { return (first_row(ck) * p.H + h) * p.dA * 2 + (NH == 2 ? ck.h * DA * 2 : 0); };
   auto rowsB = [&](const Chunk& ck) { return ((first_row(ck) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
 
   if (!state_role) {
@@ -251,7 +271,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     };
     auto feed_load = [&](FeedRegs& fr, const Chunk& c2) {
       const bool live = c2.ok && !(dbg & 1);
-      const uint32_t lenA = (live && !STATE) ? (uint32_t)(c2.L - 1) * rowA + p.dA * 2 : 0u;
+      const uint32_t lenA = (live && !STATE) ? (uint32_t)(c2.L - 1) * rowA + DA * 2 : 0u;
       const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
       const bool sf = SFX && c2.sfx;
       const fprt::BufView xv = fprt::make_buf((sf ? Xsg : Xg) + (live ? rowsA(c2) : 0), lenA);
@@ -301,9 +321,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     feed_store_z(fa, 0);
     fprt::block_sync();   // stage 0 is filled
 
-    // One chunk.  `refill` is the register set freed by the previous iteration (it receives chunk
-    // it + 2), `ready` holds chunk it + 1.  Returns false after the last chunk.
-    auto iteration = [&](int it, FeedRegs& refill, const FeedRegs& ready) -> bool {
+    // One item.  `refill` is the register set freed by the previous iteration (it receives item
+    // it + 2), `ready` holds item it + 1.  Returns false after the last item.  `half` is the
+    // parity of `it` as a type: with NH = 2 the first visit of a chunk opens the accumulators and
+    // the second closes them; with NH = 1 every visit does both.
+    f32x16 yacc, sd, so;
+    auto iteration = [&](auto half, int it, FeedRegs& refill, const FeedRegs& ready) -> bool {
+      constexpr int HF = decltype(half)::value;
+      constexpr bool opens = NH == 1 || HF == 0, closes = NH == 1 || HF == 1;
       const int s = it & 1;
       const int L = ck.L;
       const Chunk ck2 = chunk_after(ck1);
@@ -351,7 +376,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       fprt::sched_fence();
 
       // ---- phase 1: read-out of the carried state, Y^T[n][i] = sum_a R[a][n] X[i][a]
-      f32x16 yacc = {0};
+      if (opens) yacc = f32x16{0};
 #pragma unroll
       for (int t = 0; t < KS; ++t) yacc = fprt::mfma_32x32x16_bf16(rf[t], xf[t], yacc);
       fprt::sched_fence();
@@ -361,12 +386,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       // W tile takes over the registers of the R fragments); X of chunk it + 1 goes to the other stage
 #pragma unroll
       for (int t = 0; t < KS; ++t) wo[t] = ld128(ws + wo_off + 16 * t);
+      if (closes) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        zd[t] = ld_token_frag(zt + zd_off + 16 * t);
-        zo[t] = ld_token_frag(zt + zo_off + 16 * t);
+        for (int t = 0; t < 2; ++t) {
+          zd[t] = ld_token_frag(zt + zd_off + 16 * t);
+          zo[t] = ld_token_frag(zt + zo_off + 16 * t);
+        }
       }
-      f32x16 sd = {0};
+      if (opens) sd = f32x16{0};
 #pragma unroll
       for (int t = 0; t < KS; ++t) sd = fprt::mfma_32x32x16_bf16(wd[t], xf[t], sd);
       feed_store_x(ready, s ^ 1);
@@ -377,23 +404,32 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       // tile converted in its shadow, and Z of chunk it + 1 is transposed into the other stage.
       // Accumulator element r = 8 t + e is token 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the
       // order the Z fragments are read in.
-      f32x16 so = {0};
+      if (opens) so = f32x16{0};
 #pragma unroll
       for (int t = 0; t < KS; ++t) so = fprt::mfma_32x32x16_bf16(wo[t], xf[t], so);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) yacc[r] *= wread;
       u32x4 pd[2], po[2];
+      if (closes) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+        for (int r = 0; r < 16; ++r) yacc[r] *= wread;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 8 * t + 2 * e;
-          pd[t][e] = fprt::pack_bf16x2(sd[r] * mw_d[r], sd[r + 1] * mw_d[r + 1]) & keep_d[4 * t + e];
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 8 * t + 2 * e;
+            pd[t][e] = fprt::pack_bf16x2(sd[r] * mw_d[r], sd[r + 1] * mw_d[r + 1]) & keep_d[4 * t + e];
+          }
         }
       }
       feed_store_z(ready, s ^ 1);
       fprt::sched_fence();
       fprt::prof_stamp(it, 3);
+      if (!closes) {   // first half of the contraction: nothing to finish yet
+        fprt::block_sync();
+        ckp = no_chunk;
+        ck = ck1;
+        ck1 = ck2;
+        return true;
+      }
 
       // ---- phase 4: Y^T += Z^T P^T
 #pragma unroll
@@ -429,8 +465,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       return ck.ok;
     };
     for (int it = 0;; it += 2) {
-      if (!iteration(it, fa, fb)) break;
-      if (!iteration(it + 1, fb, fa)) break;
+      if (!iteration(Half<0>{}, it, fa, fb)) break;
+      if (!iteration(Half<1>{}, it + 1, fb, fa)) break;
     }
     return;
   }
@@ -468,16 +504,19 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   auto prefetch = [&](ChunkRegs& cr, const Chunk& ck) {
     // views that start at the chunk's first row and end with its last: later rows read as zero
     const bool live = ck.ok && !(dbg & 1);
-    const uint32_t lenA = live ? (uint32_t)(ck.L - 1) * rowA + p.dA * 2 : 0u;
+    const uint32_t lenA = live ? (uint32_t)(ck.L - 1) * rowA + DA * 2 : 0u;
     const fprt::BufView wb = fprt::make_buf(((SFX && ck.sfx) ? Wsg : Wg) + (live ? rowsA(ck) : 0), lenA);
 #pragma unroll
     for (int r = 0; r < 4; ++r) cr.w[r] = fprt::buf_load128(wb, wg_off[r]);
   };
 
-  // state tiles: racc[nn] is R[32 ablk + acc_row][32 (nb0 + nn) + c]
-  f32x16 racc[NNW];
+  // state tiles: racc[hf][nn] is R[DA hf + 32 ablk + acc_row][32 (nb0 + nn) + c]
+  f32x16 racc[NH][NNW];
 #pragma unroll
-  for (int nn = 0; nn < NNW; ++nn) racc[nn] = f32x16{0};
+  for (int hf = 0; hf < NH; ++hf) {
+#pragma unroll
+    for (int nn = 0; nn < NNW; ++nn) racc[hf][nn] = f32x16{0};
+  }
 
   // ---- this wave's tile of a state matrix <-> global memory --------------------------------
   // Global accesses are 16 bytes per lane along the contiguous direction of the matrix; the
@@ -513,14 +552,16 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       tile_soff[u] = stage_elem(n_l * 32 + 8 * piece);
     }
   }
+  // byte offset of half hf of the rows of R inside a state matrix
+  const uint32_t half_stride = 2u * DA * (uint32_t)(tposed ? 1 : p.rs_a);
   // issue the global loads of a tile; `src` null or !live -> zeros without memory traffic
-  auto tile_load = [&](TileRegs& tr, const uint16_t* src, bool live) {
+  auto tile_load = [&](TileRegs& tr, const uint16_t* src, bool live, int hf) {
     const fprt::BufView view = fprt::make_buf(src, (src && live) ? (uint32_t)(mat * 2) : 0u);
 #pragma unroll
-    for (int u = 0; u < NP; ++u) tr.v[u] = fprt::buf_load128(view, tile_goff[u]);
+    for (int u = 0; u < NP; ++u) tr.v[u] = fprt::buf_load128(view, tile_goff[u] + hf * half_stride);
   };
   // R (+)= loaded tile, through stage s
-  auto tile_accumulate = [&](const TileRegs& tr, int s, bool add) {
+  auto tile_accumulate = [&](const TileRegs& tr, int s, bool add, f32x16 (&racc)[NNW]) {
     uint16_t* st = RT + s * BV * RT_LD;
 #pragma unroll
     for (int u = 0; u < NP; ++u) st128(st + tile_soff[u], tr.v[u]);
@@ -549,7 +590,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     fprt::wave_sync();   // the staging area is reused right after
   };
   // bf16(R) -> global matrix at dst, through stage s
-  auto tile_store = [&](uint16_t* dst, int s) {
+  auto tile_store = [&](uint16_t* dst, int s, const f32x16 (&racc)[NNW], int hf) {
     uint16_t* st = RT + s * BV * RT_LD;
 #pragma unroll
     for (int nn = 0; nn < NNW; ++nn) {
@@ -570,7 +611,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     fprt::wave_sync();
     const fprt::BufView view = fprt::make_buf(dst, (uint32_t)(mat * 2));
 #pragma unroll
-    for (int u = 0; u < NP; ++u) fprt::buf_store128(view, tile_goff[u], ld128(st + tile_soff[u]));
+    for (int u = 0; u < NP; ++u) fprt::buf_store128(view, tile_goff[u] + hf * half_stride, ld128(st + tile_soff[u]));
     fprt::wave_sync();   // the staging area is reused right after
   };
   // block-state matrix of the block that ends at token t1 (its gradient in a reverse pass)
@@ -581,7 +622,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   auto ends_block = [&](int t1) { return bs > 0 && (t1 % bs) == 0; };
 
   // bf16 copy of R -> LDS stage s
-  auto write_rt = [&](int s) {
+  auto write_rt = [&](int s, const f32x16 (&racc)[NNW]) {
     uint16_t* rt = RT + s * BV * RT_LD;
 #pragma unroll
     for (int nn = 0; nn < NNW; ++nn) {
@@ -631,16 +672,17 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   Chunk cur = first_chunk(slot), nxt = chunk_after(cur);
   prefetch(setA, cur);
   if (DEEP) prefetch(setB, nxt);
-  {
+#pragma unroll
+  for (int hf = 0; hf < NH; ++hf) {
     // initial R, plus the gradient of the last block state if the first chunk of a reverse pass ends a block
     TileRegs t_init, t_inj;
-    tile_load(t_init, p.R0 ? state_matrix(p.R0, cur.b) : nullptr, true);
+    tile_load(t_init, p.R0 ? state_matrix(p.R0, cur.b) : nullptr, true, hf);
     const bool inj = BLOCKS && p.Bin && ends_block(cur.t0 + cur.L);
-    tile_load(t_inj, inj ? block_matrix(p.Bin, cur.b, cur.t0 + cur.L) : nullptr, inj);
-    if (p.R0) tile_accumulate(t_init, 0, false);
-    if (inj) tile_accumulate(t_inj, 0, true);
+    tile_load(t_inj, inj ? block_matrix(p.Bin, cur.b, cur.t0 + cur.L) : nullptr, inj, hf);
+    if (p.R0) tile_accumulate(t_init, 0, false, racc[hf]);
+    if (inj) tile_accumulate(t_inj, 0, true, racc[hf]);
   }
-  write_rt(0);
+  write_rt(0, racc[0]);
   store_transposed(setA, cur);
   store_rowmajor(setA, 0);
   if (!DEEP) prefetch(setA, nxt);
@@ -649,20 +691,27 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   int Lg_cached = -1;
   float gL = 1.f;
   // One iteration: `refill` is the register set freed by the previous iteration (it receives
-  // chunk it + 2), `ready` holds chunk it + 1.  Returns false after the last chunk.
-  auto iteration = [&](int it, ChunkRegs& refill, const ChunkRegs& ready) -> bool {
+  // item it + 2), `ready` holds item it + 1.  Returns false after the last item.  `half` is the
+  // parity of `it` as a type; with NH = 2 it is the half of R this visit updates.
+  auto iteration = [&](auto half, int it, ChunkRegs& refill, const ChunkRegs& ready) -> bool {
+    constexpr int HF = NH == 2 ? decltype(half)::value : 0;
+    constexpr bool closes = HF == NH - 1;   // the chunk is complete after this visit
+    f32x16 (&racc_h)[NNW] = racc[HF];
     const int s = it & 1;
     fprt::prof_stamp(it, 0);
     const Chunk nn = chunk_after(nxt);
     if (DEEP) prefetch(refill, nn);
     // gradient of the block state that the next chunk ends (reverse pass); an empty view otherwise
-    const bool inj = BLOCKS && p.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
-    TileRegs t_inj;
-    if (BLOCKS) tile_load(t_inj, inj ? block_matrix(p.Bin, nxt.b, nxt.t0 + nxt.L) : nullptr, inj);
+    const bool inj = BLOCKS && closes && p.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
+    TileRegs t_inj[NH];
+    if (BLOCKS && closes) {
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf) tile_load(t_inj[hf], inj ? block_matrix(p.Bin, nxt.b, nxt.t0 + nxt.L) : nullptr, inj, hf);
+    }
     // initial state of the next sequence, if the next chunk starts one
     const bool fresh = MULTI && nxt.ok && nxt.first;
     TileRegs t_init;
-    if (MULTI) tile_load(t_init, (fresh && p.R0) ? state_matrix(p.R0, nxt.b) : nullptr, fresh);
+    if (MULTI) tile_load(t_init, (fresh && p.R0) ? state_matrix(p.R0, nxt.b) : nullptr, fresh, 0);
 
     if (dbg & 4) {
       fprt::block_sync();
@@ -700,7 +749,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 #pragma unroll
       for (int nq = 0; nq < NNW; ++nq) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) racc[nq][r] *= gL;
+        for (int r = 0; r < 16; ++r) racc_h[nq][r] *= gL;
       }
     }
     fprt::sched_fence();
@@ -712,7 +761,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     for (int kt = 0; kt < 2; ++kt) {
       if (kt < nk) {
 #pragma unroll
-        for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[kt], zlo[nq][kt], racc[nq]);
+        for (int nq = 0; nq < NNW; ++nq) racc_h[nq] = fprt::mfma_32x32x16_bf16(wf[kt], zlo[nq][kt], racc_h[nq]);
       }
     }
 #pragma unroll
@@ -732,7 +781,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     for (int kt = 0; kt < 2; ++kt) {
       if (2 + kt < nk) {
 #pragma unroll
-        for (int nq = 0; nq < NNW; ++nq) racc[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc[nq]);
+        for (int nq = 0; nq < NNW; ++nq) racc_h[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc_h[nq]);
       }
     }
     store_rowmajor(ready, s ^ 1);
@@ -744,20 +793,30 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // over, and the bf16 copy for the next chunk's read-out is written.  All of them use this
     // wave's part of the other stage's R buffer, in this order.
     const int t1 = cur.t0 + cur.L;
-    if (BLOCKS && p.Bout && ends_block(t1)) tile_store(const_cast<uint16_t*>(block_matrix(p.Bout, cur.b, t1)), s ^ 1);
-    if (cur.last && p.Rout) tile_store(const_cast<uint16_t*>(state_matrix(p.Rout, cur.b)), s ^ 1);
+    if (closes) {
+#pragma unroll
+      for (int hf = 0; hf < NH; ++hf) {
+        if (BLOCKS && p.Bout && ends_block(t1))
+          tile_store(const_cast<uint16_t*>(block_matrix(p.Bout, cur.b, t1)), s ^ 1, racc[hf], hf);
+        if (cur.last && p.Rout) tile_store(const_cast<uint16_t*>(state_matrix(p.Rout, cur.b)), s ^ 1, racc[hf], hf);
+      }
+    }
     fprt::prof_stamp(it, 3);
     if (nxt.ok) {
       if (MULTI && fresh) {
         if (p.R0) {
-          tile_accumulate(t_init, s ^ 1, false);
+          tile_accumulate(t_init, s ^ 1, false, racc[0]);
         } else {
 #pragma unroll
-          for (int nq = 0; nq < NNW; ++nq) racc[nq] = f32x16{0};
+          for (int nq = 0; nq < NNW; ++nq) racc[0][nq] = f32x16{0};
         }
       }
-      if (BLOCKS && inj) tile_accumulate(t_inj, s ^ 1, true);
-      if (!STATE) write_rt(s ^ 1);
+      if (BLOCKS && closes && inj) {
+#pragma unroll
+        for (int hf = 0; hf < NH; ++hf) tile_accumulate(t_inj[hf], s ^ 1, true, racc[hf]);
+      }
+      // the next visit reads the other half (NH = 2), which this visit did not touch
+      if (!STATE) write_rt(s ^ 1, racc[(HF + 1) % NH]);
     }
     fprt::prof_stamp(it, 4);
     fprt::block_sync();
@@ -768,8 +827,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     return true;
   };
   for (int it = 0;; it += 2) {
-    if (!iteration(it, setA, DEEP ? setB : setA)) break;
-    if (!iteration(it + 1, DEEP ? setB : setA, setA)) break;
+    if (!iteration(Half<0>{}, it, setA, DEEP ? setB : setA)) break;
+    if (!iteration(Half<1>{}, it + 1, DEEP ? setB : setA, setA)) break;
   }
 }
 

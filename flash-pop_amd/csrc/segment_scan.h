@@ -2,7 +2,7 @@
 // (batch, head) state matrix through the S segments in fp32.
 #pragma once
 #include "pass_args.h"
-#include "retention_pass.h"   // bf16 helpers
+#include "lds_access.h"
 
 namespace fpk {
 

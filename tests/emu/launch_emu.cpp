@@ -1,7 +1,6 @@
 // CPU implementation of fpk_launch_pass: runs the kernel bodies with one OS thread per GPU
 // lane, workgroups one after another.  Test infrastructure only.
 #include "device_rt.h"
-#include "retention_pass.h"
 #include "retention_pass_ws.h"
 #include "segment_scan.h"
 #include "decode_step.h"
@@ -68,7 +67,7 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
     return 1;
   }
   if (multi && (!ws || blocks || suffix)) {
-    *err = "several batch entries per workgroup need the plain wave-specialised kernel";
+    *err = "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
     return 1;
   }
   const int nwg = a.slots * a.H * (a.dB / fpk::BV);
@@ -86,7 +85,8 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
       if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_MULTI>(a, l); });
       return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_PLAIN>(a, l); });
     case 256:
-      return run_grid(fpk::NTHREADS, nwg, fpk::lds_bytes(256), [&](char* l) { fpk::retention_pass<256>(a, l); });
+      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_BLOCKS, 2>(a, l); });
+      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_PLAIN, 2>(a, l); });
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }

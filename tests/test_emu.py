@@ -31,7 +31,8 @@ def _check_all(pairs):
     (1, 150, 2, 128, 128, 0.5),     # ragged tail, initial state
     (1, 100, 2, 64, 128, None),     # dk != dv, no initial state
     (2, 64, 1, 128, 64, 0.0),       # exactly one chunk, zero state
-    (1, 70, 1, 256, 64, 0.3),       # widest contraction
+    (1, 70, 1, 256, 64, 0.3),       # widest contraction (two visits per chunk), state stored as it is
+    (1, 100, 1, 64, 256, 0.3),      # widest contraction in the dq and dk passes, state read transposed
     (1, 5, 3, 64, 64, 0.5),         # shorter than a chunk
     (5, 16, 1, 128, 128, 0.5),      # several short sequences per workgroup (suffix-like), odd count
     (4, 100, 1, 64, 128, None),     # several multi-chunk sequences per workgroup, no initial state
@@ -52,6 +53,7 @@ def test_plain_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std):
     (2, 28, 1, 64, 64, 15),         # block < chunk
     (1, 130, 1, 64, 64, 32),        # block divides chunk
     (1, 40, 1, 64, 64, 100),        # no full block at all
+    (1, 130, 1, 256, 64, 32),       # widest contraction with block states written and their gradients read
 ])
 def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
     decays = oracle.head_decays(H, (5, 12))
