@@ -1,4 +1,4 @@
-"""The committed golden vectors (tests/golden/retention_golden.npz, float64 closed form on seeded
+"""The committed golden vectors (tests/golden/*.npz, float64 closed forms on seeded
 bf16-representable inputs) against the oracle on the CPU and against the HIP ops on the GPU."""
 import os
 
@@ -54,3 +54,43 @@ def test_hip_ops_match_golden(gold):
     hp.assert_close(blocks, gold["blocks"], "blocks", head_dim=2)
     for name, leaf in zip(("pop_dq", "pop_dk", "pop_dv", "pop_ds0"), leaves):
         hp.assert_close(leaf.grad, gold[name], name, head_dim=1 if name == "pop_ds0" else 2)
+
+
+FUSED_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "pop_fused_golden.npz")
+FUSED_INPUTS = ("q", "k", "v", "s0", "q_sfx", "k_sfx", "v_sfx")
+FUSED_GRADS = ("dq", "dk", "dv", "ds0", "dq_sfx", "dk_sfx", "dv_sfx")
+
+
+@pytest.fixture(scope="module")
+def gold_fused():
+    z = np.load(FUSED_PATH, allow_pickle=False)
+    g = {k: torch.from_numpy(z[k]) for k in z.files}
+    g["decays"] = tuple(float(x) for x in z["decays"])
+    g["block"] = int(z["block"])
+    return g
+
+
+def test_oracle_matches_fused_pop_golden(gold_fused):
+    g = gold_fused
+    q, k, v, s0, qs, ks, vs = ins = [g[n].double().requires_grad_() for n in FUSED_INPUTS]
+    o, o_sfx, last = oracle.pop_fused_retention(q, k, v, s0, qs, ks, vs, g["decays"], g["block"])
+    for name, got in (("o", o), ("o_sfx", o_sfx), ("last", last)):
+        assert torch.allclose(got.float(), g[name], rtol=1e-5, atol=1e-5), name
+    loss = (o * g["d_o"].double()).sum() + (o_sfx * g["d_o_sfx"].double()).sum() + (last * g["d_last"].double()).sum()
+    for name, got in zip(FUSED_GRADS, torch.autograd.grad(loss, ins)):
+        assert torch.allclose(got.float(), g[name], rtol=1e-5, atol=1e-4), name
+
+
+@pytest.mark.gpu
+def test_fused_pop_op_matches_golden(gold_fused):
+    from flash_pop_amd import flash_pop_retention_with_suffixes
+    g = gold_fused
+    bf = lambda n: g[n].to(torch.bfloat16).to("cuda:0")
+    q, k, v, s0, qs, ks, vs = leaves = [bf(n).requires_grad_() for n in FUSED_INPUTS]
+    o, o_sfx, last = flash_pop_retention_with_suffixes(q, k, v, s0, g["decays"], g["block"], qs, ks, vs)
+    torch.autograd.backward([o, o_sfx, last], [bf("d_o"), bf("d_o_sfx"), bf("d_last")])
+    hp.assert_close(o, g["o"], "o", head_dim=2)
+    hp.assert_close(o_sfx, g["o_sfx"], "o_sfx", head_dim=2)
+    hp.assert_close(last, g["last"], "last", head_dim=1)
+    for name, leaf in zip(FUSED_GRADS, leaves):
+        hp.assert_close(leaf.grad, g[name], name, head_dim=1 if name == "ds0" else 2)
