@@ -53,9 +53,9 @@ class HipBackend:
         from flash_pop_amd import flash_pop_retention_with_suffixes
         return flash_pop_retention_with_suffixes(q, k, v, s, decays, block, q_s, k_s, v_s)
 
-    def step(self, q, k, v, s, decays):
+    def step(self, q, k, v, s, decays, in_place=False):
         from flash_pop_amd import retention_recurrent
-        return retention_recurrent(q, k, v, decays, s)
+        return retention_recurrent(q, k, v, decays, s, in_place=in_place)
 
 
 class OracleBackend:
@@ -73,7 +73,7 @@ class OracleBackend:
         o, o_s, last = oracle.pop_fused_retention(f(q), f(k), f(v), f(s), f(q_s), f(k_s), f(v_s), decays, block)
         return o.to(q.dtype), o_s.to(q.dtype), last.to(q.dtype)
 
-    def step(self, q, k, v, s, decays):
+    def step(self, q, k, v, s, decays, in_place=False):
         import oracle
         o, S = oracle.recurrent_step(q.float(), k.float(), v.float(), None if s is None else s.float(), decays)
         return o.to(q.dtype), S.to(q.dtype)
@@ -166,12 +166,14 @@ class Layer(nn.Module):
         o, state = backend.plain(q, k, v, state, r.decays)
         return self._ffn(x + r.finish(xn, o)), state
 
-    def recurrent(self, backend, x, index, state):
-        """x [B, D], one token (flash_pop/retnet.py:325-366, 493-512)."""
+    def recurrent(self, backend, x, index, state, in_place=False):
+        """x [B, D], one token at position `index` (an int, or a one-element tensor on the device)
+        (flash_pop/retnet.py:325-366, 493-512)."""
         r = self.retention
         xn = self._norm(self.norm1, x)
-        q, k, v = r.qkv(xn[:, None], torch.full((1,), index, device=x.device))
-        o, state = backend.step(q[:, 0], k[:, 0], v[:, 0], state, r.decays)
+        pos = index if isinstance(index, torch.Tensor) else torch.full((1,), index, device=x.device)
+        q, k, v = r.qkv(xn[:, None], pos)
+        o, state = backend.step(q[:, 0], k[:, 0], v[:, 0], state, r.decays, in_place=in_place)
         return self._ffn(x + r.finish(xn, o)), state
 
 
@@ -211,14 +213,53 @@ class PopRetNetLM(nn.Module):
         return self._logits(x), new_states
 
     @torch.no_grad()
-    def recurrent(self, backend, token, states: List, index: int):
+    def recurrent(self, backend, token, states: List, index, in_place=False):
         """One decode step: token [B] -> (logits [B, vocab], new states)."""
         x = self.embed(token)
         new_states = []
         for layer, st in zip(self.layers, states):
-            x, st = layer.recurrent(backend, x, index, st)
+            x, st = layer.recurrent(backend, x, index, st, in_place)
             new_states.append(st)
         return self._logits(x), new_states
+
+
+class GraphedGreedyDecoder:
+    """Greedy decoding with one decode step captured in a HIP graph: the step is a chain of small
+    launches (12 layers of projections, norms and the decode-step kernel), so replaying it as a
+    graph removes the per-launch host cost.  Everything the step reads or writes lives in fixed
+    buffers: the token, the position, the per-layer states (updated in place) and the logits."""
+
+    def __init__(self, model: PopRetNetLM, backend, states: List, token: torch.Tensor, index: int):
+        self.model, self.backend = model, backend
+        self.states = [s.clone().contiguous() for s in states]
+        self.token = token.clone()
+        self.pos = torch.full((1,), index, device=token.device, dtype=torch.long)
+        self.logits = None
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):            # warm-up outside the capture: lazy initialisation, autotuning
+            keep = [s.clone() for s in self.states], self.token.clone(), self.pos.clone()
+            for _ in range(2):
+                self._step()
+            for dst, src in zip(self.states, keep[0]):
+                dst.copy_(src)
+            self.token.copy_(keep[1])
+            self.pos.copy_(keep[2])
+        torch.cuda.current_stream().wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self._step()
+
+    def _step(self):
+        logits, _ = self.model.recurrent(self.backend, self.token, self.states, self.pos, in_place=True)
+        self.logits = logits
+        self.token.copy_(logits.argmax(-1))
+        self.pos.add_(1)
+
+    def step(self):
+        """Advance by one token; returns the logits buffer (overwritten by the next step)."""
+        self.graph.replay()
+        return self.logits
 
 
 def build(cfg: HarnessConfig, seed: int, device) -> PopRetNetLM:

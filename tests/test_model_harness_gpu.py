@@ -67,3 +67,33 @@ def test_recurrent_decode_continues_the_pop_states():
     r = _ratio(torch.stack(outs, dim=1), full_logits[:, T:])
     _say(f"[model] decode vs chunkwise logits, RMS ratio {r:.4f}")
     assert r < 3e-2
+
+
+def test_graph_captured_decode_step_equals_eager():
+    """One decode step captured in a HIP graph and replayed 12 times, with eager work and
+    synchronisations between the replays; every replay is compared with the eager decode loop."""
+    cfg = mh.HarnessConfig(**SMALL)
+    B, T, steps = 2, 64, 12
+    backend = mh.HipBackend()
+    model = mh.build(cfg, seed=13, device=DEV).eval()
+    g = torch.Generator().manual_seed(6)
+    tokens = torch.randint(0, cfg.vocab, (B, T), generator=g).to(DEV)
+    with torch.no_grad():
+        _, states = model.chunkwise(backend, tokens)
+        first = tokens[:, -1].clone()
+        eager_logits, eager_tokens, st, tok = [], [], [s.clone() for s in states], first
+        for i in range(steps):
+            logits, st = model.recurrent(backend, tok, st, T + i)
+            tok = logits.argmax(-1)
+            eager_logits.append(logits.clone())
+            eager_tokens.append(tok.clone())
+        dec = mh.GraphedGreedyDecoder(model, backend, states, first, T)
+        for i in range(steps):
+            logits = dec.step().clone()
+            torch.cuda.synchronize()
+            scratch = torch.randn(256, 256, device=DEV) @ torch.randn(256, 256, device=DEV)   # unrelated eager work
+            torch.cuda.synchronize()
+            assert torch.equal(logits, eager_logits[i]), f"replay {i}: logits differ from the eager step"
+            assert torch.equal(dec.token, eager_tokens[i]), f"replay {i}"
+            del scratch
+        assert int(dec.pos.item()) == T + steps
