@@ -1,12 +1,15 @@
 #!/bin/bash
-# Collects the rocprofv3 evidence for the pass kernels on BASELINE configs 2 and 4 (run from the repo
+# Collects the rocprofv3 evidence for the pass kernels on benchmark configurations 2 and 4 (run from the repo
 # root on a GPU box): kernel-trace statistics, then hardware counters in separate passes (one
 # counter group per run), then the same HBM counters on a plain copy of known size for scaling.
-# Raw output goes to gpurun_out/profile/; the figures are summarised by hand into profiles/.
+# Raw output goes to the directory given as the first argument; the figures are summarised by
+# hand into profiles/.
+#   usage: flash-pop_amd/profile_counters.sh <output directory>
 set -e
 R=$(cd "$(dirname "$0")/.." && pwd)
-O=$R/gpurun_out/profile
-mkdir -p "$O"
+[ -n "$1" ] || { echo "usage: $0 <output directory>" >&2; exit 2; }
+mkdir -p "$1"
+O=$(cd "$1" && pwd)
 cd /tmp && export TMPDIR=/tmp
 BENCH="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu --no-long --no-model"
 COPY="python3 $R/bench.py --copy-calibration"

@@ -10,7 +10,7 @@ import oracle
 
 BF16 = torch.bfloat16
 
-# BASELINE tolerance for bf16 (rtol = atol = 2e-2) and the reference's own bar for outputs and
+# Stated tolerance for bf16 (rtol = atol = 2e-2) and the reference's own bar for outputs and
 # states, RMS(err)/RMS(ref) < 0.005 (tests/test_fused_retention.py:119,131).
 RTOL = 2e-2
 ATOL = 2e-2

@@ -120,6 +120,6 @@ def test_fused_argument_errors():
 
 
 def test_config4_fused():
-    """BASELINE config 4 in one walk: B8 H16 d128, T4096 in 64-token blocks, 65 suffixes of 16 tokens
+    """Benchmark configuration 4 in one walk: B8 H16 d128, T4096 in 64-token blocks, 65 suffixes of 16 tokens
     per sequence.  Oracle on one sequence."""
     run_fused(8, 64, 64, 16, 16, 128, 128, 0.05, seed=40, oracle_batches=[5])

@@ -245,7 +245,7 @@ def test_pop_fused_is_the_composition_and_pins_last_state():
 
 
 def test_fp32_matches_fp64_at_config1():
-    """BASELINE config 1 (fp32, B1 H4 T512 d64, chunk 64, no initial state): the fp32 oracle
+    """Benchmark configuration 1 (fp32, B1 H4 T512 d64, chunk 64, no initial state): the fp32 oracle
     is within 1e-4 of the float64 closed form."""
     decays = oracle.head_decays(4)
     q, k, v, _ = rand_inputs(1, 512, 4, 64, 64, False, dtype=torch.float32, seed=0)

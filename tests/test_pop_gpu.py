@@ -111,6 +111,6 @@ def test_pop_suffix_path_small():
 
 
 def test_config4_pop_with_suffixes():
-    """BASELINE config 4: B8 H16 d128, T4096 in 64-token blocks, 16-token suffixes at every boundary
+    """Benchmark configuration 4: B8 H16 d128, T4096 in 64-token blocks, 16-token suffixes at every boundary
     (N + 1 = 65 per sequence, the first from S0).  Oracle on one sequence."""
     _suffix_case(B=8, N=64, block=64, Ls=16, H=16, dk=128, dv=128, seed=40, oracle_batches=[5])

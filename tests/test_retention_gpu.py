@@ -62,14 +62,14 @@ def test_decay_range_of_reference_tests():
 
 
 def test_config2_headline_shape():
-    """BASELINE config 2 at full size: B8 H16 T4096 d128, zero initial state, dS_final = 0.
+    """Benchmark configuration 2 at full size: B8 H16 T4096 d128, zero initial state, dS_final = 0.
     Oracle on two batch entries (streams are independent); the rest is covered by invariants."""
     o, S, grads = run_plain(8, 4096, 16, 128, 128, 0.0, seed=0, with_ds=False, oracle_batches=[0, 7])
     assert all(torch.isfinite(t.float()).all() for t in (o, S, *grads))
 
 
 def test_config3_long_context_carried_state():
-    """BASELINE config 3: B2 H8 T16384 dk128 dv256, S0 ~ N(0, 0.02^2), gradient of the final state too."""
+    """Benchmark configuration 3: B2 H8 T16384 dk128 dv256, S0 ~ N(0, 0.02^2), gradient of the final state too."""
     run_plain(2, 16384, 8, 128, 256, 0.02, seed=3, with_ds=True, oracle_batches=[1])
 
 
