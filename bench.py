@@ -1,7 +1,7 @@
 """Benchmark of the retention hot path on one MI355X.
 
 A step is one forward + backward of fused_chunk_retention over one synthetic batch of
-Benchmark configuration 2 (bf16, B=8 H=16 T=4096 dk=dv=128, zero initial state, dO ~ N(0,1)), inputs
+benchmark configuration 2 (bf16, B=8 H=16 T=4096 dk=dv=128, zero initial state, dO ~ N(0,1)), inputs
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic FLOP count
 (dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the pass kernel measured
 with events on the launch stream, and the CPU oracle timed on the host cores beside it.
