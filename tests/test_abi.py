@@ -80,3 +80,31 @@ def test_python_wrappers_refuse_cpu_tensors():
         fused_chunk_retention(q.float(), q.float(), q.float(), None, (0.9, 0.9))
     with pytest.raises(AssertionError, match="head decays"):
         fused_chunk_retention(q, q, q, None, (0.9,))
+
+
+def test_new_entry_points_check_their_arguments(lib):
+    dec = (ctypes.c_double * 2)(0.9, 0.95)
+    p, null = ctypes.c_void_p(0x1000), None
+    # decode step: shape, NULL and dimension checks come before any launch
+    assert lib.fp_retention_decode_step(p, p, p, null, dec, p, null, 1, 2, 64, 64, None) == -1
+    assert lib.fp_retention_decode_step(p, p, p, null, dec, p, p, 1, 2, 64, 96, None) == -3
+    assert lib.fp_retention_decode_step(p, p, p, null, dec, p, p, 0, 2, 64, 64, None) == -2
+    # split entry points: same checks as the plain ones, and an invalid shape needs no workspace
+    assert lib.fp_retention_workspace_bytes(0, 64, 2, 64, 64) == 0
+    assert lib.fp_retention_workspace_bytes(1, 64, 2, 96, 64) == 0
+    assert lib.fp_retention_fwd_split(null, p, p, null, dec, p, null, 1, 8, 2, 64, 64, null, 0, None) == -1
+    assert lib.fp_retention_bwd_split(p, p, p, null, dec, null, null, p, p, p, null, 1, 8, 2, 64, 64, null, 0, None) == -1
+
+
+def test_new_python_wrappers_refuse_cpu_tensors():
+    import torch
+    from flash_pop_amd import flash_pop_retention_with_suffixes, retention_recurrent
+    q = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
+    sfx = torch.zeros(3, 2, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        flash_pop_retention_with_suffixes(q, q, q, None, (0.9, 0.9), 4, sfx, sfx, sfx)
+    x = torch.zeros(1, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        retention_recurrent(x, x, x, (0.9, 0.9), None)
+    with pytest.raises(ValueError, match=r"\[B,H,dk\]"):
+        retention_recurrent(x[0], x[0], x[0], (0.9, 0.9), None)
