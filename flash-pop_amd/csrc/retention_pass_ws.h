@@ -9,12 +9,15 @@
 //                         -> Y tile into LDS.  2 x 2 grid: `ib` = 32 chunk rows, `nb` = 32 columns.
 //                         Branch-free: every wave computes both 32 x 32 score tiles of its rows;
 //                         the tile outside the decay window is cleared after conversion.
-//                         They also feed X and Z: bounds-checked buffer loads two chunks ahead in
-//                         registers, X copied and Z transposed into LDS, and they store the Y tile
-//                         of the previous chunk.
-//   state waves   (4..7)  the W traffic (loads two chunks ahead, row-major copy and the weighted
-//                         transpose into LDS), the state update R = gamma^L R + (wkey W)^T Z in
-//                         fp32 accumulators and its bf16 copy for the read-out, block states.
+//                         They also feed X and Z: bounds-checked buffer loads into registers, X
+//                         copied and Z transposed into LDS one chunk ahead, and they store the Y
+//                         tile of the previous chunk.
+//   state waves   (4..7)  the W traffic (loads, row-major copy and the weighted transpose into
+//                         LDS), the state update R = gamma^L R + (wkey W)^T Z in fp32
+//                         accumulators and its bf16 copy for the read-out, block states.
+// Each role has one set of load registers: as soon as chunk i + 1 has gone from it into LDS
+// (during chunk i), the loads of chunk i + 2 are issued into it, in the shadow of the MFMAs; they
+// have a whole chunk time to arrive.  (A second set, loaded a chunk earlier, was slower.)
 // The split keeps the two roles' instruction streams about equally long.
 //
 // LDS tiles are double-buffered: while the readout waves work on chunk i from stage i & 1 the
@@ -263,21 +266,23 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const int y_row = tid >> 2, y_col = (tid & 3) * 16;
     const uint32_t yg_off = y_row * rowB + y_col * 2;
 
-    // Two register sets, so that the loads run two chunks ahead.  Loads and stores are issued
-    // unconditionally (zero-length views when there is nothing to do): exact wait counts.
+    // Loads and stores are issued unconditionally (zero-length views when there is nothing to
+    // do): exact wait counts.
     struct FeedRegs {
       u32x4 x[NXP];
       u32x2 z[4];
     };
-    auto feed_load = [&](FeedRegs& fr, const Chunk& c2) {
-      const bool live = c2.ok && !(dbg & 1);
-      const uint32_t lenA = (live && !STATE) ? (uint32_t)(c2.L - 1) * rowA + DA * 2 : 0u;
-      const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
-      const bool sf = SFX && c2.sfx;
-      const fprt::BufView xv = fprt::make_buf((sf ? Xsg : Xg) + (live ? rowsA(c2) : 0), lenA);
-      const fprt::BufView zv = fprt::make_buf((sf ? Zsg : Zg) + (live ? rowsB(c2) : 0), lenB);
+    auto feed_load_x = [&](FeedRegs& fr, const Chunk& c2) {
+      const bool live = c2.ok && !(dbg & 1) && !STATE;
+      const uint32_t lenA = live ? (uint32_t)(c2.L - 1) * rowA + DA * 2 : 0u;
+      const fprt::BufView xv = fprt::make_buf(((SFX && c2.sfx) ? Xsg : Xg) + (live ? rowsA(c2) : 0), lenA);
 #pragma unroll
       for (int u = 0; u < NXP; ++u) fr.x[u] = fprt::buf_load128(xv, xg_off[u]);
+    };
+    auto feed_load_z = [&](FeedRegs& fr, const Chunk& c2) {
+      const bool live = c2.ok && !(dbg & 1);
+      const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
+      const fprt::BufView zv = fprt::make_buf(((SFX && c2.sfx) ? Zsg : Zg) + (live ? rowsB(c2) : 0), lenB);
 #pragma unroll
       for (int r = 0; r < 4; ++r) fr.z[r] = fprt::buf_load64(zv, zg_off[r]);
     };
@@ -314,25 +319,26 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     };
 
     Chunk ck = first_chunk(slot), ck1 = chunk_after(ck), ckp = no_chunk;
-    FeedRegs fa, fb;
-    feed_load(fa, ck);
-    feed_load(fb, ck1);
-    feed_store_x(fa, 0);
-    feed_store_z(fa, 0);
-    fprt::block_sync();   // stage 0 is filled
+    FeedRegs feed;
+    feed_load_x(feed, ck);
+    feed_load_z(feed, ck);
+    feed_store_x(feed, 0);
+    feed_store_z(feed, 0);
+    feed_load_x(feed, ck1);
+    feed_load_z(feed, ck1);
+    fprt::block_sync();   // stage 0 is filled, item 1 is on its way
 
-    // One item.  `refill` is the register set freed by the previous iteration (it receives item
-    // it + 2), `ready` holds item it + 1.  Returns false after the last item.  `half` is the
-    // parity of `it` as a type: with NH = 2 the first visit of a chunk opens the accumulators and
-    // the second closes them; with NH = 1 every visit does both.
+    // One item.  `feed` holds item it + 1 on entry; once its parts have gone into LDS they are
+    // reloaded with item it + 2.  Returns false after the last item.  `half` is the parity of `it`
+    // as a type: with NH = 2 the first visit of a chunk opens the accumulators and the second
+    // closes them; with NH = 1 every visit does both.
     f32x16 yacc, sd, so;
-    auto iteration = [&](auto half, int it, FeedRegs& refill, const FeedRegs& ready) -> bool {
+    auto iteration = [&](auto half, int it) -> bool {
       constexpr int HF = decltype(half)::value;
       constexpr bool opens = NH == 1 || HF == 0, closes = NH == 1 || HF == 1;
       const int s = it & 1;
       const int L = ck.L;
       const Chunk ck2 = chunk_after(ck1);
-      feed_load(refill, ck2);
       if (!STATE) drain_y(ckp, s ^ 1);
       const uint16_t* xs = XS + s * CH * X_LD;
       const uint16_t* ws = WS + s * CH * X_LD;
@@ -350,7 +356,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 
       fprt::prof_stamp(it, 0);
       if (STATE) {   // feed Z for the state waves, nothing else
-        feed_store_z(ready, s ^ 1);
+        feed_store_z(feed, s ^ 1);
+      feed_load_z(feed, ck2);
         fprt::block_sync();
         ckp = ck;
         ck = ck1;
@@ -396,7 +403,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       if (opens) sd = f32x16{0};
 #pragma unroll
       for (int t = 0; t < KS; ++t) sd = fprt::mfma_32x32x16_bf16(wd[t], xf[t], sd);
-      feed_store_x(ready, s ^ 1);
+      feed_store_x(feed, s ^ 1);
+      feed_load_x(feed, ck2);
       fprt::sched_fence();
       fprt::prof_stamp(it, 2);
 
@@ -420,7 +428,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
           }
         }
       }
-      feed_store_z(ready, s ^ 1);
+      feed_store_z(feed, s ^ 1);
+      feed_load_z(feed, ck2);
       fprt::sched_fence();
       fprt::prof_stamp(it, 3);
       if (!closes) {   // first half of the contraction: nothing to finish yet
@@ -465,8 +474,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       return ck.ok;
     };
     for (int it = 0;; it += 2) {
-      if (!iteration(Half<0>{}, it, fa, fb)) break;
-      if (!iteration(Half<1>{}, it + 1, fb, fa)) break;
+      if (!iteration(Half<0>{}, it)) break;
+      if (!iteration(Half<1>{}, it + 1)) break;
     }
     return;
   }
@@ -491,14 +500,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const int ws_off = (4 * w_tg) * X_LD + 32 * ablk + 8 * w_fg;
   const int wt_off = (8 * w_fg) * T_LD + 4 * w_tg;
 
-  // Two register sets of loaded chunks, so that global loads run two chunks ahead of the math.
-  // The block-state instantiation needs the registers of the second set for the block-state
-  // tile in flight and keeps its loads one chunk ahead instead.
-  constexpr bool DEEP = true;
   struct ChunkRegs {
     u32x4 w[4];
   };
-  ChunkRegs setA, setB;
+  ChunkRegs wregs;
   // Loads are issued unconditionally so that the number of outstanding memory operations is the
   // same in every iteration; a chunk that does not exist gets zero-length views (no traffic).
   auto prefetch = [&](ChunkRegs& cr, const Chunk& ck) {
@@ -670,8 +675,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 
   // ---- prologue: chunk 0 into stage 0, chunk 1 in flight ----------------------------------
   Chunk cur = first_chunk(slot), nxt = chunk_after(cur);
-  prefetch(setA, cur);
-  if (DEEP) prefetch(setB, nxt);
+  prefetch(wregs, cur);
 #pragma unroll
   for (int hf = 0; hf < NH; ++hf) {
     // initial R, plus the gradient of the last block state if the first chunk of a reverse pass ends a block
@@ -683,24 +687,23 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (inj) tile_accumulate(t_inj, 0, true, racc[hf]);
   }
   write_rt(0, racc[0]);
-  store_transposed(setA, cur);
-  store_rowmajor(setA, 0);
-  if (!DEEP) prefetch(setA, nxt);
+  store_transposed(wregs, cur);
+  store_rowmajor(wregs, 0);
+  prefetch(wregs, nxt);
   fprt::block_sync();
 
   int Lg_cached = -1;
   float gL = 1.f;
-  // One iteration: `refill` is the register set freed by the previous iteration (it receives
-  // item it + 2), `ready` holds item it + 1.  Returns false after the last item.  `half` is the
-  // parity of `it` as a type; with NH = 2 it is the half of R this visit updates.
-  auto iteration = [&](auto half, int it, ChunkRegs& refill, const ChunkRegs& ready) -> bool {
+  // One iteration: `wregs` holds the W rows of item it + 1 on entry and is reloaded with item
+  // it + 2 once they have gone into LDS.  Returns false after the last item.  `half` is the parity
+  // of `it` as a type; with NH = 2 it is the half of R this visit updates.
+  auto iteration = [&](auto half, int it) -> bool {
     constexpr int HF = NH == 2 ? decltype(half)::value : 0;
     constexpr bool closes = HF == NH - 1;   // the chunk is complete after this visit
     f32x16 (&racc_h)[NNW] = racc[HF];
     const int s = it & 1;
     fprt::prof_stamp(it, 0);
     const Chunk nn = chunk_after(nxt);
-    if (DEEP) prefetch(refill, nn);
     // gradient of the block state that the next chunk ends (reverse pass); an empty view otherwise
     const bool inj = BLOCKS && closes && p.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
     TileRegs t_inj[NH];
@@ -772,7 +775,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
           zhi[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * (2 + kt) + 4 * g);
       }
     }
-    store_transposed(ready, nxt);
+    store_transposed(wregs, nxt);
     fprt::sched_fence();
     fprt::prof_stamp(it, 2);
 
@@ -784,8 +787,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         for (int nq = 0; nq < NNW; ++nq) racc_h[nq] = fprt::mfma_32x32x16_bf16(wf[2 + kt], zhi[nq][kt], racc_h[nq]);
       }
     }
-    store_rowmajor(ready, s ^ 1);
-    if (!DEEP) prefetch(refill, nn);   // refill and ready are the same set here
+    store_rowmajor(wregs, s ^ 1);
+    prefetch(wregs, nn);
     fprt::sched_fence();
 
     // ---- phase 3: the state after a full block or at the end of a sequence leaves, the gradient
@@ -827,8 +830,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     return true;
   };
   for (int it = 0;; it += 2) {
-    if (!iteration(Half<0>{}, it, setA, DEEP ? setB : setA)) break;
-    if (!iteration(Half<1>{}, it + 1, DEEP ? setB : setA, setA)) break;
+    if (!iteration(Half<0>{}, it)) break;
+    if (!iteration(Half<1>{}, it + 1)) break;
   }
 }
 
