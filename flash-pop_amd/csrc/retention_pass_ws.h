@@ -112,7 +112,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const int slot = (wg / ntile) / p.H;   // first batch entry of this workgroup
 
   const int dbg = fprt::dbg_flags();   // always 0 outside profiling builds
-  const int T = p.T, bs = p.block;
+  const int T = p.T;
+  const int bs = (BLOCKS || SFX) ? p.block : 0;   // only these walks cut chunks at block boundaries
   const bool rev = p.reverse != 0;
   const float lg = p.log2g[h];
 
@@ -147,8 +148,13 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     bool sfx;               // a suffix (t0 is its block boundary) rather than a context chunk
     int n;                  // WALK_SUFFIX only: index of the suffix, or of the context chunk's block
     int h;                  // NH = 2 only: which half of the contraction this visit covers
+    uint32_t row;           // index of the item's first row among all rows of its tensor
   };
-  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0, 0};
+  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0, 0, 0u};
+  auto with_row = [&](Chunk ck) {
+    ck.row = (SFX && ck.sfx) ? ((uint32_t)ck.b * (p.nblk + 1) + ck.n) * p.Ls : (uint32_t)ck.b * T + ck.t0;
+    return ck;
+  };
   auto first_chunk = [&](int b) {
     Chunk ck = {b, 0, 0, b < p.B, true, false, false, 0};
     if (ck.ok) {
@@ -162,7 +168,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         ck.last = !has_more(next_pos(ck.t0, ck.L));
       }
     }
-    return ck;
+    return with_row(ck);
   };
   auto chunk_after = [&](const Chunk& ck) {
     if (!ck.ok) return ck;
@@ -193,21 +199,20 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
           n.n = m; n.t0 = pos - CH > lo ? pos - CH : lo; n.L = pos - n.t0;
         }
       }
-      return n;
+      return with_row(n);
     }
     chunk_at(next_pos(ck.t0, ck.L), n.t0, n.L);
     n.last = !has_more(next_pos(n.t0, n.L));
-    return n;
+    return with_row(n);
   };
 
   const uint32_t rowA = (uint32_t)p.H * p.dA * 2, rowB = (uint32_t)p.H * p.dB * 2;   // row pitch in bytes
   // byte offset of the item's first row for head h in an [B,T,H,dA] tensor (suffixes:
-  // [B, nblk + 1, Ls, H, dA]), resp. of this tile's columns in the dB-wide tensors
-  auto first_row = [&](const Chunk& ck) {
-    return (SFX && ck.sfx) ? ((size_t)ck.b * (p.nblk + 1) + ck.n) * p.Ls : (size_t)ck.b * T + ck.t0;
-  };
-  auto rowsA = [&](const Chunk& ck) { return (first_row(ck) * p.H + h) * p.dA * 2 + (NH == 2 ? ck.h * DA * 2 : 0); };
-  auto rowsB = [&](const Chunk& ck) { return ((first_row(ck) * p.H + h) * p.dB + (size_t)tile * BV) * 2; };
+  // [B, nblk + 1, Ls, H, dA]), resp. of this tile's columns in the dB-wide tensors: one 32 x 32 -> 64
+  // bit multiply each (a tensor has fewer than 2^32 rows)
+  const uint32_t headA = (uint32_t)h * p.dA * 2, headB = ((uint32_t)h * p.dB + (uint32_t)tile * BV) * 2;
+  auto rowsA = [&](const Chunk& ck) { return (size_t)ck.row * rowA + headA + (NH == 2 ? ck.h * DA * 2 : 0); };
+  auto rowsB = [&](const Chunk& ck) { return (size_t)ck.row * rowB + headB; };
 
   if (!state_role) {
     // =============================== readout waves ===============================
@@ -621,7 +626,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   };
   // block-state matrix of the block that ends at token t1 (its gradient in a reverse pass)
   auto block_matrix = [&](const uint16_t* base, int b, int t1) {
-    return base + (((size_t)b * p.nblk + (t1 / bs - 1)) * p.H + h) * mat;
+    const int m = bs > 0 ? t1 / bs - 1 : 0;   // bs is a compile-time 0 in the walks that never get here
+    return base + (((size_t)b * p.nblk + m) * p.H + h) * mat;
   };
   auto state_matrix = [&](const uint16_t* base, int b) { return base + ((size_t)b * p.H + h) * mat; };
   auto ends_block = [&](int t1) { return bs > 0 && (t1 % bs) == 0; };
