@@ -1,0 +1,109 @@
+// Runs every C entry point on the CPU thread harness with heap buffers of exactly the sizes the
+// header documents, for AddressSanitizer / UBSan builds: any access of a kernel body outside a
+// tensor, the workspace or the LDS block it was given aborts the run.  Test infrastructure only.
+#include "../../include/flashpop_hip.h"
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+namespace {
+
+std::vector<void*> g_live;
+
+uint16_t* buf(size_t n, bool fill = true) {
+  uint16_t* p = static_cast<uint16_t*>(malloc(n * 2 + (n == 0)));
+  for (size_t i = 0; i < n; ++i) p[i] = fill ? static_cast<uint16_t>(0x3c00 + (rand() & 0x1ff)) : 0;   // bf16 in [1, 2)
+  g_live.push_back(p);
+  return p;
+}
+
+int done(int rc, const char* what, int B, int T, int H, int dk, int dv, int extra) {
+  for (void* p : g_live) free(p);
+  g_live.clear();
+  if (rc) {
+    printf("FAILED %s: %s\n", what, fp_last_error());
+  } else {
+    printf("ok %s B%d T%d H%d dk%d dv%d (%d)\n", what, B, T, H, dk, dv, extra);
+  }
+  fflush(stdout);
+  return rc;
+}
+
+int plain(int B, int T, int H, int dk, int dv, bool split) {
+  std::vector<double> dec(H, 0.97);
+  const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
+  uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = buf(ns), *o = buf(nv, false), *so = buf(ns, false);
+  uint16_t *dO = buf(nv), *dS = buf(ns), *dq = buf(nq, false), *dk_ = buf(nq, false), *dv_ = buf(nv, false), *ds0 = buf(ns, false);
+  int rc;
+  if (split) {
+    const size_t wb = fp_retention_workspace_bytes(B, T, H, dk, dv);
+    void* ws = wb ? aligned_alloc(16, wb) : nullptr;
+    rc = fp_retention_fwd_split(q, k, v, s, dec.data(), o, so, B, T, H, dk, dv, ws, wb, nullptr);
+    if (!rc) rc = fp_retention_bwd_split(q, k, v, s, dec.data(), dO, dS, dq, dk_, dv_, ds0, B, T, H, dk, dv, ws, wb, nullptr);
+    free(ws);
+    return done(rc, "split", B, T, H, dk, dv, (int)wb);
+  }
+  rc = fp_retention_fwd(q, k, v, s, dec.data(), o, so, B, T, H, dk, dv, nullptr);
+  if (!rc) rc = fp_retention_bwd(q, k, v, s, dec.data(), dO, dS, dq, dk_, dv_, ds0, B, T, H, dk, dv, nullptr);
+  return done(rc, "plain", B, T, H, dk, dv, 0);
+}
+
+int pop(int B, int T, int H, int dk, int dv, int block) {
+  std::vector<double> dec(H, 0.97);
+  const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
+  const int nb = T / block;
+  uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = buf(ns), *o = buf(nv, false), *dO = buf(nv);
+  uint16_t *dq = buf(nq, false), *dk_ = buf(nq, false), *dv_ = buf(nv, false), *ds0 = buf(ns, false);
+  uint16_t *bs = buf(nb * ns, false), *dbs = buf(nb * ns);
+  int rc = fp_pop_retention_fwd(q, k, v, s, dec.data(), o, nb ? bs : nullptr, B, T, H, dk, dv, block, nullptr);
+  if (!rc) rc = fp_pop_retention_bwd(q, k, v, s, dec.data(), dO, nb ? dbs : nullptr, dq, dk_, dv_, ds0, B, T, H, dk, dv, block, nullptr);
+  return done(rc, "pop", B, T, H, dk, dv, block);
+}
+
+int fused(int B, int nblk, int block, int ls, int H, int dk, int dv) {
+  std::vector<double> dec(H, 0.97);
+  const int T = nblk * block;
+  const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
+  const size_t sq = (size_t)B * (nblk + 1) * ls * H * dk, sv = (size_t)B * (nblk + 1) * ls * H * dv;
+  uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = buf(ns), *qs = buf(sq), *ks = buf(sq), *vs = buf(sv);
+  uint16_t *o = buf(nv, false), *os = buf(sv, false), *so = buf(ns, false), *dO = buf(nv), *dOs = buf(sv), *dS = buf(ns);
+  uint16_t *dq = buf(nq, false), *dk_ = buf(nq, false), *dv_ = buf(nv, false), *dqs = buf(sq, false), *dks = buf(sq, false),
+           *dvs = buf(sv, false), *ds0 = buf(ns, false);
+  int rc = fp_pop_fused_fwd(q, k, v, s, qs, ks, vs, dec.data(), o, os, so, B, T, H, dk, dv, block, ls, nullptr);
+  if (!rc) rc = fp_pop_fused_bwd(q, k, v, s, qs, ks, vs, dec.data(), dO, dOs, dS, dq, dk_, dv_, dqs, dks, dvs, ds0, B, T, H,
+                                 dk, dv, block, ls, nullptr);
+  return done(rc, "fused", B, T, H, dk, dv, ls);
+}
+
+int decode(int B, int H, int dk, int dv) {
+  std::vector<double> dec(H, 0.97);
+  const size_t ns = (size_t)B * H * dk * dv;
+  uint16_t *q = buf((size_t)B * H * dk), *k = buf((size_t)B * H * dk), *v = buf((size_t)B * H * dv), *s = buf(ns);
+  uint16_t *o = buf((size_t)B * H * dv, false), *so = buf(ns, false);
+  int rc = fp_retention_decode_step(q, k, v, s, dec.data(), o, so, B, H, dk, dv, nullptr);
+  if (!rc) rc = fp_retention_decode_step(q, k, v, so, dec.data(), o, so, B, H, dk, dv, nullptr);   // in place
+  return done(rc, "decode", B, 1, H, dk, dv, 0);
+}
+
+}  // namespace
+
+int main() {
+  int rc = 0;
+  rc |= plain(5, 16, 1, 128, 128, false);     // several short sequences per workgroup
+  rc |= plain(3, 70, 2, 64, 64, false);       // ragged tails
+  rc |= plain(2, 1, 1, 64, 64, false);        // single token
+  rc |= plain(1, 65, 1, 64, 256, false);      // two visits per chunk, state read transposed
+  rc |= plain(1, 130, 1, 256, 64, false);     // two visits per chunk, state as stored
+  rc |= plain(1, 512, 1, 64, 128, true);      // cut into segments (state-only walk, scan)
+  rc |= pop(1, 287, 1, 64, 128, 144);
+  rc |= pop(2, 28, 1, 64, 64, 15);
+  rc |= pop(1, 40, 1, 64, 64, 100);           // no full block
+  rc |= pop(1, 96, 1, 256, 64, 32);           // block states with two visits per chunk
+  rc |= fused(2, 2, 80, 5, 1, 64, 128);
+  rc |= fused(1, 3, 24, 64, 1, 128, 64);
+  rc |= decode(2, 3, 64, 128);
+  rc |= decode(1, 1, 256, 256);
+  return rc;
+}
