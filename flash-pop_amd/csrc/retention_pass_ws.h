@@ -237,7 +237,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       const int d1 = rev ? (acc_row(2 * e + 1, g) - c) : (c - acc_row(2 * e + 1, g));
       keep_d[e] = (d0 >= 0 ? 0x0000ffffu : 0u) | (d1 >= 0 ? 0xffff0000u : 0u);
     }
-    const uint32_t keep_o = other_live ? 0xffffffffu : 0u;
     const int i_row = 32 * ib + c;                 // this lane's chunk row (query index)
     const int x_off = i_row * X_LD + 8 * g;
     const int wd_off = (32 * ib + c) * X_LD + 8 * g;
@@ -338,8 +337,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // as a type: with NH = 2 the first visit of a chunk opens the accumulators and the second
     // closes them; with NH = 1 every visit does both.
     f32x16 yacc, sd, so;
-    auto iteration = [&](auto half, int it) -> bool {
+    auto iteration = [&](auto half, auto with_other, int it) -> bool {
       constexpr int HF = decltype(half)::value;
+      constexpr bool OTHER = decltype(with_other)::value;   // false: the other tile is outside the decay window
       constexpr bool opens = NH == 1 || HF == 0, closes = NH == 1 || HF == 1;
       const int s = it & 1;
       const int L = ck.L;
@@ -396,13 +396,15 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
 
       // ---- phase 2: scores^T of the diagonal tile; the other W tile and Z arrive meanwhile (the
       // W tile takes over the registers of the R fragments); X of chunk it + 1 goes to the other stage
+      if (OTHER) {
 #pragma unroll
-      for (int t = 0; t < KS; ++t) wo[t] = ld128(ws + wo_off + 16 * t);
+        for (int t = 0; t < KS; ++t) wo[t] = ld128(ws + wo_off + 16 * t);
+      }
       if (closes) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           zd[t] = ld_token_frag(zt + zd_off + 16 * t);
-          zo[t] = ld_token_frag(zt + zo_off + 16 * t);
+          if (OTHER) zo[t] = ld_token_frag(zt + zo_off + 16 * t);
         }
       }
       if (opens) sd = f32x16{0};
@@ -418,8 +420,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       // Accumulator element r = 8 t + e is token 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the
       // order the Z fragments are read in.
       if (opens) so = f32x16{0};
+      if (OTHER) {
 #pragma unroll
-      for (int t = 0; t < KS; ++t) so = fprt::mfma_32x32x16_bf16(wo[t], xf[t], so);
+        for (int t = 0; t < KS; ++t) so = fprt::mfma_32x32x16_bf16(wo[t], xf[t], so);
+      }
       u32x4 pd[2], po[2];
       if (closes) {
 #pragma unroll
@@ -448,16 +452,18 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       // ---- phase 4: Y^T += Z^T P^T
 #pragma unroll
       for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zd[t], pd[t], yacc);
+      if (OTHER) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2; ++t) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 8 * t + 2 * e;
-          po[t][e] = fprt::pack_bf16x2(so[r] * mw_o[r], so[r + 1] * mw_o[r + 1]) & keep_o;
+          for (int e = 0; e < 4; ++e) {
+            const int r = 8 * t + 2 * e;
+            po[t][e] = fprt::pack_bf16x2(so[r] * mw_o[r], so[r + 1] * mw_o[r + 1]);
+          }
         }
-      }
 #pragma unroll
-      for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zo[t], po[t], yacc);
+        for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zo[t], po[t], yacc);
+      }
       fprt::sched_fence();
 
       // accumulator element r holds column n = 32 nb + 8 (r / 4) + 4 g + r % 4 of row i_row
@@ -478,9 +484,17 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       if (!ck.ok) drain_y(ckp, s);   // the last Y tile
       return ck.ok;
     };
-    for (int it = 0;; it += 2) {
-      if (!iteration(Half<0>{}, it)) break;
-      if (!iteration(Half<1>{}, it + 1)) break;
+    // Two copies of the loop, chosen once: the waves whose other tile is dead run the one without it.
+    if (other_live) {
+      for (int it = 0;; it += 2) {
+        if (!iteration(Half<0>{}, Half<1>{}, it)) break;
+        if (!iteration(Half<1>{}, Half<1>{}, it + 1)) break;
+      }
+    } else {
+      for (int it = 0;; it += 2) {
+        if (!iteration(Half<0>{}, Half<0>{}, it)) break;
+        if (!iteration(Half<1>{}, Half<0>{}, it + 1)) break;
+      }
     }
     return;
   }
