@@ -7,8 +7,10 @@
 //
 //   readout waves (0..3)  scores^T = W X^T -> P (bf16, in registers) ; Y^T = wread (R X^T) + Z^T P^T
 //                         -> Y tile into LDS.  2 x 2 grid: `ib` = 32 chunk rows, `nb` = 32 columns.
-//                         Branch-free: every wave computes both 32 x 32 score tiles of its rows;
-//                         the tile outside the decay window is cleared after conversion.
+//                         A wave's rows meet two 32 x 32 score tiles: the diagonal one, whose
+//                         masked half is cleared after conversion, and one that lies wholly inside
+//                         or wholly outside the decay window.  The loop has no data-dependent
+//                         branches; it exists in two copies, with and without the second tile.
 //                         They also feed X and Z: bounds-checked buffer loads into registers, X
 //                         copied and Z transposed into LDS one chunk ahead, and they store the Y
 //                         tile of the previous chunk.
@@ -69,7 +71,6 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 //              the readout waves feed Z and do nothing else, X is not read and Y not written.
 enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WALK_STATE = 4 };
 
-//
 // NH = 2 handles a contraction width of 2 DA (p.dA = 256 with DA = 128) with the LDS footprint of
 // DA: every chunk is visited twice, once per half of the columns of X and W (of the rows of R).
 // Scores and read-out are sums over the contraction index, so the readout waves simply keep
@@ -87,7 +88,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   constexpr int YB_LD = BV + 8;
   constexpr int KS = DA / 16;       // MFMA k-steps over dA
   constexpr int FG = DA / 8;        // 16-byte pieces per X row
-  constexpr int NXP = CH * FG / 256;  // X pieces per state thread
+  constexpr int NXP = CH * FG / 256;  // X pieces per readout thread
   constexpr int NAB = DA / 32;      // 32-row blocks of R: 2 or 4
   constexpr int NNW = NAB == 4 ? 2 : 1;   // 32-column blocks of R per state wave
 
