@@ -274,7 +274,7 @@ def model_leg(args, dev):
     }
 
 
-def cpu_leg(sample_batch=1, reps=2):
+def cpu_leg(sample_batch=8, reps=2):
     """The oracle (chunk 64, fp32, torch autograd for the backward) on the host cores, on
     `sample_batch` of the 8 sequences of config 2."""
     import torch
