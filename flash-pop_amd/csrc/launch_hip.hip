@@ -1,4 +1,6 @@
 // gfx950 entry points of the pass kernels and the launcher the C-ABI layer calls.
+#include <atomic>
+
 #include "device_rt.h"
 #include "retention_pass_ws.h"
 #include "segment_scan.h"
@@ -22,23 +24,30 @@ __global__ __launch_bounds__(fpk::DECODE_THREADS) void decode_step_kernel(const 
   fpk::decode_step(args, lds);
 }
 
+// LDS above 64 KB has to be opted into once per device and kernel.  One bit per kernel (`slot`)
+// and device, shared by all threads of the process: once any thread has run a kernel on a device,
+// no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
+// launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
+constexpr int kMaxDevices = 64;
+std::atomic<uint32_t> g_armed[kMaxDevices];
+
 template <typename Kernel>
-int launch(Kernel kernel, int threads, int lds, int* armed_device, const fpk::PassArgs& a, hipStream_t stream,
+int launch(Kernel kernel, int threads, int lds, int slot, const fpk::PassArgs& a, hipStream_t stream,
            const char** err) {
-  // LDS above 64 KB has to be opted into, once per device and kernel.
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     *err = "hipGetDevice failed";
     return 1;
   }
-  if (*armed_device != dev) {
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1u << slot))) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
         hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    *armed_device = dev;
+    if (tracked) g_armed[dev].fetch_or(1u << slot, std::memory_order_release);
   }
   const int nwg = a.slots * a.H * (a.dB / fpk::BV);
   hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a);
@@ -77,7 +86,6 @@ int fpk_compute_units() {
 
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  static thread_local int armed[12] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
   fpk::PassArgs a = args;
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool ws = a.dA == 64 || a.dA == 128;
@@ -114,20 +122,20 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   }
   switch (a.dA) {
     case 64:
-      if (suffix) return launch(retention_pass_ws_kernel<64, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[7], a, s, err);
-      if (blocks) return launch(retention_pass_ws_kernel<64, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[0], a, s, err);
-      if (a.state_only) return launch(retention_pass_ws_kernel<64, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[9], a, s, err);
-      if (multi) return launch(retention_pass_ws_kernel<64, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[1], a, s, err);
-      return launch(retention_pass_ws_kernel<64, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), &armed[2], a, s, err);
+      if (suffix) return launch(retention_pass_ws_kernel<64, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 7, a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<64, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 0, a, s, err);
+      if (a.state_only) return launch(retention_pass_ws_kernel<64, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 9, a, s, err);
+      if (multi) return launch(retention_pass_ws_kernel<64, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 1, a, s, err);
+      return launch(retention_pass_ws_kernel<64, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 2, a, s, err);
     case 128:
-      if (suffix) return launch(retention_pass_ws_kernel<128, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[8], a, s, err);
-      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[3], a, s, err);
-      if (a.state_only) return launch(retention_pass_ws_kernel<128, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[10], a, s, err);
-      if (multi) return launch(retention_pass_ws_kernel<128, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[4], a, s, err);
-      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[5], a, s, err);
+      if (suffix) return launch(retention_pass_ws_kernel<128, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 8, a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 3, a, s, err);
+      if (a.state_only) return launch(retention_pass_ws_kernel<128, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 10, a, s, err);
+      if (multi) return launch(retention_pass_ws_kernel<128, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 4, a, s, err);
+      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 5, a, s, err);
     case 256:   // two visits per chunk, 128 of the 256 contraction columns each
-      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[6], a, s, err);
-      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), &armed[11], a, s, err);
+      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 6, a, s, err);
+      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 11, a, s, err);
     default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
   }
 }
