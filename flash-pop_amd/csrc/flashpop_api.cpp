@@ -51,6 +51,8 @@ int check_shape(const Shape& s, const double* decays) {
   // the kernels address one (batch, head) stream with 32-bit byte offsets
   const long long span = 2LL * s.T * s.H * (s.dk > s.dv ? s.dk : s.dv);
   if (span >= (1LL << 32)) return fail(FP_ERR_BAD_SHAPE, "T * H * max(dk, dv) too large: one sequence must stay below 4 GiB");
+  // ... and a row of a tensor by a 32-bit index
+  if ((long long)s.B * s.T >= (1LL << 32)) return fail(FP_ERR_BAD_SHAPE, "B * T too large: a tensor must have fewer than 2^32 rows");
   const long long wgs = (long long)s.B * s.H * ((s.dk > s.dv ? s.dk : s.dv) / fpk::BV);
   if (wgs > 0x7fffffffLL) return fail(FP_ERR_BAD_SHAPE, "B * H too large");
   for (int h = 0; h < s.H; ++h) {
@@ -293,6 +295,8 @@ int check_fused(const Shape& s, int block, int sfx_len) {
     return fail(FP_ERR_BAD_SHAPE, "suffix length must be in 1..%d (got %d)", fpk::CH, sfx_len);
   if (s.dk > 128 || s.dv > 128)
     return fail(FP_ERR_UNSUPPORTED_DIM, "the fused POP op supports dk and dv of 64 or 128 (got dk=%d, dv=%d)", s.dk, s.dv);
+  if ((long long)s.B * (s.T / block + 1) * sfx_len >= (1LL << 32))
+    return fail(FP_ERR_BAD_SHAPE, "too many suffix rows: B * (T / block_size + 1) * sfx_len must stay below 2^32");
   return FP_OK;
 }
 

@@ -279,3 +279,28 @@ def test_ops_replay_from_a_hip_graph():
         for i, (a, b) in enumerate(zip(outs, eager)):
             assert torch.equal(a, b), f"replay {replay}, output {i}"
         del filler
+
+
+def test_tensors_beyond_4_gib():
+    """136 sequences of 8192 tokens: every tensor is 4.6 GB, so row offsets need all 64 bits, and the
+    4352 (batch, head, tile) streams are walked by 256 resident workgroups, 17 sequences each.  Inputs
+    are generated on the device; the oracle runs on the first and the last sequence."""
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, d = 136, 8192, 16, 128
+    _say(f"[large] B{B} T{T} H{H} d{d}: {B * T * H * d * 2 / 2**30:.2f} GiB per tensor")
+    decays = oracle.head_decays(H)
+    g = torch.Generator(device=DEV).manual_seed(123)
+    leaves = [torch.randn(B, T, H, d, device=DEV, dtype=torch.bfloat16, generator=g).requires_grad_() for _ in range(3)]
+    s = (torch.randn(B, H, d, d, device=DEV, generator=g) * 0.05).to(torch.bfloat16).requires_grad_()
+    d_o = torch.randn(B, T, H, d, device=DEV, dtype=torch.bfloat16, generator=g)
+    o, S = fused_chunk_retention(*leaves, s, decays)
+    torch.autograd.backward([o], [d_o])
+    torch.cuda.synchronize()
+    for b in (0, B - 1):
+        sl = slice(b, b + 1)
+        ins = [t.detach()[sl].cpu() for t in (*leaves, s)]
+        o_ref, S_ref, grads = hp.oracle_plain(*ins, decays, d_o[sl].cpu(), None)
+        hp.assert_close(o[sl], o_ref, f"o[b={b}]", head_dim=2)
+        hp.assert_close(S[sl], S_ref, f"S[b={b}]", head_dim=1)
+        for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), (*leaves, s), grads):
+            hp.assert_close(leaf.grad[sl], ref, f"{name}[b={b}]", head_dim=1 if name == "ds0" else 2)
