@@ -2,7 +2,7 @@
 #include <atomic>
 
 #include "device_rt.h"
-#include "retention_pass_ws.h"
+#include "pass_dispatch.h"
 #include "segment_scan.h"
 #include "decode_step.h"
 
@@ -29,6 +29,7 @@ __global__ __launch_bounds__(fpk::DECODE_THREADS) void decode_step_kernel(const 
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
+static_assert(fpk::PASS_KERNELS <= 32, "one bit per kernel instantiation");
 std::atomic<uint32_t> g_armed[kMaxDevices];
 
 template <typename Kernel>
@@ -84,60 +85,27 @@ int fpk_compute_units() {
   return cus;
 }
 
+namespace {
+
+struct DeviceRun {
+  const fpk::PassArgs& a;
+  hipStream_t stream;
+  const char** err;
+  template <int DA, int MODE, int NH>
+  int go(int slot) const {
+    return launch(retention_pass_ws_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA), slot, a, stream, err);
+  }
+};
+
+}  // namespace
+
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
-  hipStream_t s = static_cast<hipStream_t>(stream);
   fpk::PassArgs a = args;
-  const bool blocks = a.block > 0 && (a.Bout || a.Bin);
-  const bool ws = a.dA == 64 || a.dA == 128;
-  const bool suffix = a.Ls > 0;
-  if (suffix) {
-    // what the suffix walk assumes; the C-ABI layer reports these to the caller in its own words
-    if (!ws || blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > fpk::CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys) {
-      *err = "suffix walk: needs dA of 64 or 128, T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
-      return 1;
-    }
-    a.slots = a.B;
-  }
-  // One workgroup per (batch entry, head, column tile) while that fits the chip once; beyond that
-  // the plain wave-specialised kernel lets each workgroup walk several batch entries, which keeps
-  // its load pipeline full across short sequences.
-  if (a.slots <= 0) {
-    a.slots = a.B;
-    if (ws && !blocks && !suffix) {
-      const int per_slot = a.H * (a.dB / fpk::BV);
-      int fit = fpk_compute_units() / per_slot;
-      if (fit < 1) fit = 1;
-      if (fit < a.B) a.slots = fit;
-    }
-  }
-  if (a.slots > a.B) a.slots = a.B;
-  const bool multi = a.slots < a.B;
-  if (a.state_only && (!ws || blocks || suffix || !a.Rout)) {
-    *err = "state-only walk: needs dA of 64 or 128, a final-state buffer, no block states and no suffixes";
+  if (const char* why = fpk::plan_pass(a, fpk_compute_units())) {
+    *err = why;
     return 1;
   }
-  if (multi && (!ws || blocks || suffix)) {
-    *err = "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
-    return 1;
-  }
-  switch (a.dA) {
-    case 64:
-      if (suffix) return launch(retention_pass_ws_kernel<64, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 7, a, s, err);
-      if (blocks) return launch(retention_pass_ws_kernel<64, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 0, a, s, err);
-      if (a.state_only) return launch(retention_pass_ws_kernel<64, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 9, a, s, err);
-      if (multi) return launch(retention_pass_ws_kernel<64, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 1, a, s, err);
-      return launch(retention_pass_ws_kernel<64, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(64), 2, a, s, err);
-    case 128:
-      if (suffix) return launch(retention_pass_ws_kernel<128, fpk::WALK_SUFFIX>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 8, a, s, err);
-      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 3, a, s, err);
-      if (a.state_only) return launch(retention_pass_ws_kernel<128, fpk::WALK_STATE>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 10, a, s, err);
-      if (multi) return launch(retention_pass_ws_kernel<128, fpk::WALK_MULTI>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 4, a, s, err);
-      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 5, a, s, err);
-    case 256:   // two visits per chunk, 128 of the 256 contraction columns each
-      if (blocks) return launch(retention_pass_ws_kernel<128, fpk::WALK_BLOCKS, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 6, a, s, err);
-      return launch(retention_pass_ws_kernel<128, fpk::WALK_PLAIN, 2>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(128), 11, a, s, err);
-    default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
-  }
+  return fpk::dispatch_pass(a, DeviceRun{a, static_cast<hipStream_t>(stream), err});
 }
 
 int fpk_launch_scan(const fpk::ScanArgs& a, void* stream, const char** err) {

@@ -1,0 +1,70 @@
+// Validation of one pass launch and the choice of kernel instantiation, shared by the device
+// launcher and the CPU thread harness so that both take the same decisions.
+#pragma once
+#include "pass_args.h"
+#include "retention_pass_ws.h"
+
+namespace fpk {
+
+// Number of kernel instantiations `dispatch_pass` can pick from (its `slot` argument is below this).
+constexpr int PASS_KERNELS = 12;
+
+// Checks what the walks assume about `a` and chooses a.slots (workgroups per (head, column tile))
+// for a device with `compute_units` units.  Returns nullptr, or a message for the caller.
+inline const char* plan_pass(PassArgs& a, int compute_units) {
+  const bool blocks = a.block > 0 && (a.Bout || a.Bin);
+  const bool narrow = a.dA == 64 || a.dA == 128;   // one visit per chunk
+  const bool suffix = a.Ls > 0;
+  if (a.dA != 64 && a.dA != 128 && a.dA != 256) return "unsupported contraction width (dA must be 64, 128 or 256)";
+  if (a.dB < BV || a.dB % BV != 0) return "dB must be a multiple of 64";
+  if (suffix) {
+    // the C-ABI layer reports these to the caller in its own words
+    if (!narrow || blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys)
+      return "suffix walk: needs dA of 64 or 128, T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
+    a.slots = a.B;
+  }
+  // One workgroup per (batch entry, head, column tile) while that fits the chip once; beyond that
+  // the plain walk lets each workgroup take several batch entries one after another, which keeps
+  // its load pipeline full across short sequences.
+  if (a.slots <= 0) {
+    a.slots = a.B;
+    if (narrow && !blocks && !suffix) {
+      int fit = compute_units / (a.H * (a.dB / BV));
+      if (fit < 1) fit = 1;
+      if (fit < a.B) a.slots = fit;
+    }
+  }
+  if (a.slots > a.B) a.slots = a.B;
+  if (a.state_only && (!narrow || blocks || suffix || !a.Rout))
+    return "state-only walk: needs dA of 64 or 128, a final-state buffer, no block states and no suffixes";
+  if (a.slots < a.B && (!narrow || blocks || suffix))
+    return "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
+  return nullptr;
+}
+
+// Calls run.template go<DA, MODE, NH>(slot) for the instantiation a planned `a` needs; `slot`
+// numbers the instantiations 0 .. PASS_KERNELS - 1.
+template <typename Run>
+int dispatch_pass(const PassArgs& a, Run&& run) {
+  const bool blocks = a.block > 0 && (a.Bout || a.Bin);
+  const bool suffix = a.Ls > 0, multi = a.slots < a.B;
+  if (a.dA == 64) {
+    if (suffix) return run.template go<64, WALK_SUFFIX, 1>(0);
+    if (blocks) return run.template go<64, WALK_BLOCKS, 1>(1);
+    if (a.state_only) return run.template go<64, WALK_STATE, 1>(2);
+    if (multi) return run.template go<64, WALK_MULTI, 1>(3);
+    return run.template go<64, WALK_PLAIN, 1>(4);
+  }
+  if (a.dA == 128) {
+    if (suffix) return run.template go<128, WALK_SUFFIX, 1>(5);
+    if (blocks) return run.template go<128, WALK_BLOCKS, 1>(6);
+    if (a.state_only) return run.template go<128, WALK_STATE, 1>(7);
+    if (multi) return run.template go<128, WALK_MULTI, 1>(8);
+    return run.template go<128, WALK_PLAIN, 1>(9);
+  }
+  // dA = 256: two visits per chunk, 128 of the 256 contraction columns each
+  if (blocks) return run.template go<128, WALK_BLOCKS, 2>(10);
+  return run.template go<128, WALK_PLAIN, 2>(11);
+}
+
+}  // namespace fpk

@@ -1,7 +1,7 @@
 // CPU implementation of fpk_launch_pass: runs the kernel bodies with one OS thread per GPU
 // lane, workgroups one after another.  Test infrastructure only.
 #include "device_rt.h"
-#include "retention_pass_ws.h"
+#include "pass_dispatch.h"
 #include "segment_scan.h"
 #include "decode_step.h"
 
@@ -45,50 +45,26 @@ int run_grid(int nthreads, int nwg, int lds_bytes, Body body) {
 
 }  // namespace
 
+namespace {
+
+struct HarnessRun {
+  const fpk::PassArgs& a;
+  template <int DA, int MODE, int NH>
+  int go(int /*slot*/) const {
+    const int nwg = a.slots * a.H * (a.dB / fpk::BV);
+    return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(DA), [&](char* l) { fpk::retention_pass_ws<DA, MODE, NH>(a, l); });
+  }
+};
+
+}  // namespace
+
 int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** err) {
   fpk::PassArgs a = args;
-  const bool blocks = a.block > 0 && (a.Bout || a.Bin);
-  const bool ws = a.dA == 64 || a.dA == 128;
-  const bool suffix = a.Ls > 0;
-  if (suffix) {
-    if (!ws || blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > fpk::CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys) {
-      *err = "suffix walk: needs dA of 64 or 128, T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
-      return 1;
-    }
-    a.slots = a.B;
-  }
-  // Pretend the chip is tiny, so that the several-entries-per-workgroup path is exercised:
-  // at most two workgroups per (head, column tile).
-  if (a.slots <= 0) a.slots = (ws && !blocks && !suffix && a.B > 2) ? 2 : a.B;
-  if (a.slots > a.B) a.slots = a.B;
-  const bool multi = a.slots < a.B;
-  if (a.state_only && (!ws || blocks || suffix || !a.Rout)) {
-    *err = "state-only walk: needs dA of 64 or 128, a final-state buffer, no block states and no suffixes";
+  if (const char* why = fpk::plan_pass(a, fpk_compute_units())) {
+    *err = why;
     return 1;
   }
-  if (multi && (!ws || blocks || suffix)) {
-    *err = "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
-    return 1;
-  }
-  const int nwg = a.slots * a.H * (a.dB / fpk::BV);
-  switch (a.dA) {
-    case 64:
-      if (suffix) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_SUFFIX>(a, l); });
-      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_BLOCKS>(a, l); });
-      if (a.state_only) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_STATE>(a, l); });
-      if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_MULTI>(a, l); });
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(64), [&](char* l) { fpk::retention_pass_ws<64, fpk::WALK_PLAIN>(a, l); });
-    case 128:
-      if (suffix) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_SUFFIX>(a, l); });
-      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_BLOCKS>(a, l); });
-      if (a.state_only) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_STATE>(a, l); });
-      if (multi) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_MULTI>(a, l); });
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_PLAIN>(a, l); });
-    case 256:
-      if (blocks) return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_BLOCKS, 2>(a, l); });
-      return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(128), [&](char* l) { fpk::retention_pass_ws<128, fpk::WALK_PLAIN, 2>(a, l); });
-    default: *err = "unsupported contraction width (dA must be 64, 128 or 256)"; return 1;
-  }
+  return fpk::dispatch_pass(a, HarnessRun{a});
 }
 
 // Pretends the chip has 8 compute units, so that small test shapes take the paths that large
