@@ -310,3 +310,23 @@ def test_tensors_beyond_4_gib():
         hp.assert_close(S[sl], S_ref, f"S[b={b}]", head_dim=1)
         for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), (*leaves, s), grads):
             hp.assert_close(leaf.grad[sl], ref, f"{name}[b={b}]", head_dim=1 if name == "ds0" else 2)
+
+
+def test_non_finite_future_keys_do_not_reach_earlier_outputs():
+    """Keys that are inf / nan from token 70 on: the outputs of tokens 0..69 are those of the clean
+    prefix, also inside the chunk that token 70 falls into (masked scores are cleared bit-wise after
+    the conversion, not multiplied by zero).  The reference's path has the same property
+    (`.tril()` before and after the decay mask, flash_pop/fused_retention/reference.py:21-23)."""
+    from flash_pop_amd import _lib
+    lib = _lib.load()
+    B, T, H, d, t0 = 2, 100, 2, 64, 70
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=88, state_std=0.2, device=DEV)
+    k_bad = k.clone()
+    k_bad[:, t0:, 0] = float("inf")
+    k_bad[:, t0:, 1] = float("nan")
+    o_bad, _ = hp.raw_fwd(lib, q, k_bad, v, s, decays)
+    o_clean, _ = hp.raw_fwd(lib, q[:, :t0].contiguous(), k[:, :t0].contiguous(), v[:, :t0].contiguous(), s, decays)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o_bad[:, :t0].float()).all()
+    assert torch.equal(o_bad[:, :t0], o_clean)
