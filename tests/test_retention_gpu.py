@@ -51,6 +51,7 @@ def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, 
     (1, 300, 2, 128, 256, 0.02),     # config-3 head dims
     (1, 130, 2, 256, 128, 0.1),      # dk = 256
     (2, 2048, 4, 64, 128, 0.0),      # reference grads test shape (tests/test_fused_retention.py:240-282)
+    (1, 70, 128, 64, 64, 0.1),       # the largest supported head count (decays down to 1 - 2^-132, i.e. 1.0)
 ])
 def test_parity_sweep(B, T, H, dk, dv, state_std):
     run_plain(B, T, H, dk, dv, state_std, seed=T + dk)
