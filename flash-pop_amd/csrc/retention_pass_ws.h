@@ -363,7 +363,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       fprt::prof_stamp(it, 0);
       if (STATE) {   // feed Z for the state waves, nothing else
         feed_store_z(feed, s ^ 1);
-      feed_load_z(feed, ck2);
+        feed_load_z(feed, ck2);
         fprt::block_sync();
         ckp = ck;
         ck = ck1;
