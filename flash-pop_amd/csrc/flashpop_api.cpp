@@ -12,6 +12,11 @@
 // The column dimension dB is split over workgroups, the contraction dimension dA never is,
 // so no pass needs a cross-workgroup reduction.  The dq pass re-runs the state recurrence
 // instead of reading stored chunk states; the dk and dv passes each carry dS.
+//
+// The POP entry points add block states to these passes (written by fwd, their gradients read
+// by dk and dv); the fused POP entry points add the suffix tensors in the same four roles; the
+// split entry points run the passes on segments of the sequences after a state-only pass and a
+// scan; the decode step is a kernel of its own.
 #include "../../include/flashpop_hip.h"
 
 #include <cmath>
