@@ -6,7 +6,7 @@ resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic F
 (dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the pass kernel measured
 with events on the launch stream, and the CPU oracle timed on the host cores beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop] [--no-long] [--no-model]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop] [--no-long] [--no-layer] [--no-model]
 """
 import argparse
 import json
@@ -203,9 +203,59 @@ def gpu_leg(args):
             "segments_per_sequence": _lib.load().fp_retention_workspace_bytes(B3, T3, H3, dk3, dv3)
             // (4 * B3 * H3 * dk3 * dv3),
         }
+    if not args.no_layer:
+        out["layer_ops"] = layer_leg(args, dev)
     if not args.no_model:
         out["model"] = model_leg(args, dev)
     return out
+
+
+def layer_leg(args, dev):
+    """The two elementwise stages around the op at config 2's tensor shapes (B=8 T=4096 H=16 d=128):
+    time per launch and algorithmic bytes per second (every tensor once), next to the same
+    stage as eager torch (the reference's call sequence)."""
+    import torch
+    import torch.nn.functional as F
+    import model_harness as mh
+    from flash_pop_amd import XPos, gated_group_norm
+
+    B, T, H, d = 8, 4096, 16, 128
+    g = torch.Generator(device=dev).manual_seed(7)
+    q, k, r, gate, d_out = (torch.randn(B, T, H, d, generator=g, device=dev).to(torch.bfloat16) for _ in range(5))
+    gate, d_out = gate.flatten(-2), d_out.flatten(-2)
+    tensor_bytes = q.numel() * 2
+    xpos = XPos(d)
+
+    def timed(fn, n=max(5, args.steps // 2)):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    def torch_norm_gate():
+        n = F.group_norm(r.reshape(B * T, H * d).float(), H, eps=1e-6).to(torch.bfloat16).reshape(B, T, H * d)
+        return n * F.silu(gate)
+
+    rl, gl = r.clone().requires_grad_(), gate.clone().requires_grad_()
+    out = gated_group_norm(rl, gl, 1e-6)
+    rows = []
+    for name, fn, eager, tensors in (
+            ("rotary_qk_kernel", lambda: xpos(q, k, 0), lambda: (mh.rotate(q, 0), mh.rotate(k, 0)), 4),
+            ("gated_norm_fwd_kernel", lambda: gated_group_norm(r, gate, 1e-6), torch_norm_gate, 3),
+            ("gated_norm_bwd_kernel", lambda: torch.autograd.grad(out, [rl, gl], d_out, retain_graph=True), None, 5)):
+        ms = timed(fn)
+        row = {"kernel": name, "ms": round(ms, 4), "algorithmic_gbs": round(tensors * tensor_bytes / (ms * 1e-3) / 1e9, 1),
+               "hbm_frac": round(tensors * tensor_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 3)}
+        if eager is not None:
+            row["eager_torch_ms"] = round(timed(eager, n=5), 4)
+        rows.append(row)
+    return {"workload": "B=8 T=4096 H=16 d=128 bf16: q, k rotated in one launch; per-head norm + swish gate, fwd and bwd",
+            "kernels": rows}
 
 
 def model_leg(args, dev):
@@ -227,15 +277,21 @@ def model_leg(args, dev):
         loss.backward()
         return states
 
-    for _ in range(2):
-        train_step()
-    torch.cuda.synchronize()
-    n = max(3, args.steps // 10)
-    t0 = time.perf_counter()
-    for _ in range(n):
-        states = train_step()
-    torch.cuda.synchronize()
-    train_ms = (time.perf_counter() - t0) * 1e3 / n
+    def time_train():
+        for _ in range(2):
+            train_step()
+        torch.cuda.synchronize()
+        n = max(3, args.steps // 10)
+        t0 = time.perf_counter()
+        for _ in range(n):
+            states = train_step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n, states
+
+    backend = mh.HipBackend(layer_ops=False)     # rotary embedding and norm + gate as eager torch
+    eager_ms, _ = time_train()
+    backend = mh.HipBackend()
+    train_ms, states = time_train()
 
     states = [s.detach() for s in states]
     token = batch[0][:, -1]
@@ -263,8 +319,10 @@ def model_leg(args, dev):
     tokens = B * T + B * (T // cfg.block + 1) * cfg.sfx_len
     return {
         "workload": "config 5: 12-layer POP-RetNet decoder d_model=768 H=12 dk=64 dv=128 FFN=3072 vocab=32000, "
-                    "bf16, B=8 T=2048, 64-token blocks, 16-token suffixes; eager torch around the HIP retention ops",
+                    "bf16, B=8 T=2048, 64-token blocks, 16-token suffixes; eager torch around the HIP ops "
+                    "(retention, rotary embedding of q and k, per-head norm + gate)",
         "train_step_ms": round(train_ms, 2),
+        "train_step_ms_retention_ops_only": round(eager_ms, 2),
         "train_tokens_per_s": round(tokens / (train_ms * 1e-3), 1),
         "decode_steps": decode_steps,
         "decode_ms_per_step": round(graph_ms, 3),
@@ -314,6 +372,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
     ap.add_argument("--no-long", action="store_true", help="skip the long-context (config 3) timing")
+    ap.add_argument("--no-layer", action="store_true", help="skip the timing of the rotary / norm + gate kernels")
     ap.add_argument("--no-model", action="store_true", help="skip the model-level (config 5) timing")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy (scales the FETCH_SIZE / WRITE_SIZE counters)")

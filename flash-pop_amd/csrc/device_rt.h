@@ -35,6 +35,12 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 
 // 2^x for x <= 0 (v_exp_f32, ~1 ulp; results below the normal range flush to zero).
 FP_DEVICE float exp2_approx(float x) { return __builtin_amdgcn_exp2f(x); }
+// full-precision elementary functions for the elementwise kernels
+FP_DEVICE void sincos_f32(float x, float& s, float& c) { sincosf(x, &s, &c); }
+FP_DEVICE float exp_f32(float x) { return expf(x); }
+FP_DEVICE float rsqrt_f32(float x) { return 1.0f / sqrtf(x); }
+// value held by lane (this lane ^ mask) of the wave; every lane of the wave has to call it
+FP_DEVICE float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
 // Orders LDS traffic between the lanes of one wave.  The hardware executes a wave's LDS
 // instructions in order, so this only has to stop the compiler from reordering them.

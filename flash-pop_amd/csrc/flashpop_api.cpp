@@ -16,7 +16,8 @@
 // The POP entry points add block states to these passes (written by fwd, their gradients read
 // by dk and dv); the fused POP entry points add the suffix tensors in the same four roles; the
 // split entry points run the passes on segments of the sequences after a state-only pass and a
-// scan; the decode step is a kernel of its own.
+// scan; the decode step and the two elementwise stages around the op (rotary embedding of q and
+// k, per-head normalisation with the swish gate) are kernels of their own.
 #include "../../include/flashpop_hip.h"
 
 #include <cmath>
@@ -76,6 +77,7 @@ void fill_common(fpk::PassArgs& a, const Shape& s, const double* decays) {
   for (int h = 0; h < s.H; ++h) a.log2g[h] = (float)std::log2(decays[h]);
 }
 
+bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
 const uint16_t* in(const void* p) { return static_cast<const uint16_t*>(p); }
 uint16_t* out(void* p) { return static_cast<uint16_t*>(p); }
 
@@ -482,8 +484,63 @@ int fp_retention_decode_step(const void* q, const void* k, const void* v, const 
   return FP_OK;
 }
 
+int fp_rotary_qk(const void* q_in, const void* k_in, void* q_out, void* k_out, const float* theta, const long long* start,
+                 long long start0, int B, int T, int H, int d, int inverse, void* stream) {
+  if (!q_in || !q_out || !theta) return fail(FP_ERR_NULL_POINTER, "q_in, q_out and theta must not be NULL");
+  if ((k_in == nullptr) != (k_out == nullptr)) return fail(FP_ERR_NULL_POINTER, "k_in and k_out must both be given or both be NULL");
+  if (B < 1 || T < 1 || H < 1) return fail(FP_ERR_BAD_SHAPE, "B, T, H must be >= 1 (got %d, %d, %d)", B, T, H);
+  if (d < 8 || d % 8 != 0) return fail(FP_ERR_UNSUPPORTED_DIM, "the head dimension must be a multiple of 8 (got %d)", d);
+  if (misaligned(q_in) || misaligned(k_in) || misaligned(q_out) || misaligned(k_out))
+    return fail(FP_ERR_BAD_SHAPE, "q and k must be 16-byte aligned");
+  fpk::RotaryArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.q_in = in(q_in); a.k_in = in(k_in); a.q_out = out(q_out); a.k_out = out(k_out);
+  a.theta = theta; a.start = start; a.start0 = start0;
+  a.B = B; a.T = T; a.H = H; a.d = d;
+  a.sign = inverse ? -1.f : 1.f;
+  const char* msg = "";
+  if (fpk_launch_rotary(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s", msg);
+  return FP_OK;
+}
+
+namespace {
+
+int gated_norm(const void* r, const void* g, const void* d_out, void* y, void* d_r, void* d_g, long long rows, int H,
+               int dv, double eps, void* stream) {
+  if (rows < 1 || H < 1) return fail(FP_ERR_BAD_SHAPE, "rows and H must be >= 1 (got %lld, %d)", rows, H);
+  const int lanes = dv / 8;
+  if (dv < 8 || dv % 8 != 0 || lanes > 64 || (lanes & (lanes - 1)) != 0)
+    return fail(FP_ERR_UNSUPPORTED_DIM, "dv must be 8 times a power of two, at most 512 (got %d)", dv);
+  if (!(eps >= 0.0)) return fail(FP_ERR_BAD_SHAPE, "eps must be non-negative (got %g)", eps);
+  if (misaligned(r) || misaligned(g) || misaligned(d_out) || misaligned(y) || misaligned(d_r) || misaligned(d_g))
+    return fail(FP_ERR_BAD_SHAPE, "tensors must be 16-byte aligned");
+  fpk::GatedNormArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.r = in(r); a.g = in(g); a.d_out = in(d_out); a.out = out(y); a.d_r = out(d_r); a.d_g = out(d_g);
+  a.groups = rows * H;
+  a.dv = dv;
+  a.eps = (float)eps;
+  const char* msg = "";
+  if (fpk_launch_gated_norm(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s", msg);
+  return FP_OK;
+}
+
+}  // namespace
+
+int fp_gated_group_norm_fwd(const void* r, const void* g, void* out_, long long rows, int H, int dv, double eps,
+                            void* stream) {
+  if (!r || !g || !out_) return fail(FP_ERR_NULL_POINTER, "r, g and out must not be NULL");
+  return gated_norm(r, g, nullptr, out_, nullptr, nullptr, rows, H, dv, eps, stream);
+}
+
+int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, void* d_r, void* d_g, long long rows, int H,
+                            int dv, double eps, void* stream) {
+  if (!r || !g || !d_out || !d_r || !d_g) return fail(FP_ERR_NULL_POINTER, "r, g, d_out, d_r and d_g must not be NULL");
+  return gated_norm(r, g, d_out, nullptr, d_r, d_g, rows, H, dv, eps, stream);
+}
+
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1003; }
+int fp_version(void) { return 1004; }
 
 }  // extern "C"

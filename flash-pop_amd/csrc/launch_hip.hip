@@ -5,6 +5,7 @@
 #include "pass_dispatch.h"
 #include "segment_scan.h"
 #include "decode_step.h"
+#include "layer_ops.h"
 
 namespace {
 
@@ -22,6 +23,18 @@ __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const f
 __global__ __launch_bounds__(fpk::DECODE_THREADS) void decode_step_kernel(const fpk::DecodeArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   fpk::decode_step(args, lds);
+}
+
+__global__ __launch_bounds__(fpk::LAYER_THREADS) void rotary_qk_kernel(const fpk::RotaryArgs args) {
+  fpk::rotary_qk(args);
+}
+
+__global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_fwd_kernel(const fpk::GatedNormArgs args) {
+  fpk::gated_norm_fwd(args);
+}
+
+__global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(const fpk::GatedNormArgs args) {
+  fpk::gated_norm_bwd(args);
 }
 
 // LDS above 64 KB has to be opted into once per device and kernel.  One bit per kernel (`slot`)
@@ -143,4 +156,43 @@ int fpk_launch_decode(const fpk::DecodeArgs& a, void* stream, const char** err) 
     return 1;
   }
   return 0;
+}
+
+namespace {
+
+int launched(const char** err) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    *err = hipGetErrorString(e);
+    return 1;
+  }
+  return 0;
+}
+
+}  // namespace
+
+int fpk_launch_rotary(const fpk::RotaryArgs& a, void* stream, const char** err) {
+  long long blocks = 0;
+  if (const char* why = fpk::plan_rotary(a, blocks)) {
+    *err = why;
+    return 1;
+  }
+  hipLaunchKernelGGL(rotary_qk_kernel, dim3((unsigned)blocks), dim3(fpk::LAYER_THREADS), 0,
+                     static_cast<hipStream_t>(stream), a);
+  return launched(err);
+}
+
+int fpk_launch_gated_norm(const fpk::GatedNormArgs& a, void* stream, const char** err) {
+  long long blocks = 0;
+  if (const char* why = fpk::plan_gated_norm(a, blocks)) {
+    *err = why;
+    return 1;
+  }
+  if (a.out)
+    hipLaunchKernelGGL(gated_norm_fwd_kernel, dim3((unsigned)blocks), dim3(fpk::LAYER_THREADS), 0,
+                       static_cast<hipStream_t>(stream), a);
+  else
+    hipLaunchKernelGGL(gated_norm_bwd_kernel, dim3((unsigned)blocks), dim3(fpk::LAYER_THREADS), 0,
+                       static_cast<hipStream_t>(stream), a);
+  return launched(err);
 }

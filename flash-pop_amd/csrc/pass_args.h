@@ -84,6 +84,40 @@ constexpr int decode_lds_bytes(int dv) { return (DECODE_THREADS / (dv / 8)) * dv
 constexpr int SCAN_THREADS = 256;
 constexpr int SCAN_VEC = 8;   // elements per thread
 
+// Rotary position embedding of q and k in one launch.  Pairs (x[2i], x[2i+1]) of every head are
+// rotated by the angle float(position) * theta[i], `sign` = -1 rotates back (the gradient).
+// q, k [B, T, H, d] bf16 (k nullable); the position of token t of sequence b is
+// (start ? start[b] : start0) + t.  Output may alias input.
+struct RotaryArgs {
+  const uint16_t* q_in;
+  const uint16_t* k_in;    // nullable, together with k_out
+  uint16_t* q_out;
+  uint16_t* k_out;
+  const float* theta;      // [d / 2], device
+  const long long* start;  // [B], device, nullable
+  long long start0;
+  int B, T, H, d;
+  float sign;
+};
+
+// Per-head normalisation of the retention output followed by the swish gate:
+//   n = bf16((r - mean) / sqrt(var + eps))  over the dv values of one (row, head), biased variance
+//   out = bf16(n * bf16(g / (1 + exp(-g))))
+// r [rows, H, dv], g and out [rows, H * dv], bf16; statistics in fp32.  The backward launch
+// (d_out given) writes d_r and d_g instead of out.
+struct GatedNormArgs {
+  const uint16_t* r;
+  const uint16_t* g;
+  const uint16_t* d_out;   // backward only
+  uint16_t* out;           // forward only
+  uint16_t* d_r;           // backward only
+  uint16_t* d_g;           // backward only
+  long long groups;        // rows * H
+  int dv;
+  float eps;
+};
+constexpr int LAYER_THREADS = 256;
+
 }  // namespace fpk
 
 // Launches the pass kernel on `stream` (a hipStream_t, or ignored by the CPU test harness).
@@ -98,3 +132,7 @@ int fpk_compute_units();
 
 // Launches the decode-step kernel.  Same conventions as fpk_launch_pass.
 int fpk_launch_decode(const fpk::DecodeArgs& args, void* stream, const char** err);
+
+// Launch the rotary kernel / the gated per-head normalisation (forward if a.out, else backward).
+int fpk_launch_rotary(const fpk::RotaryArgs& args, void* stream, const char** err);
+int fpk_launch_gated_norm(const fpk::GatedNormArgs& args, void* stream, const char** err);

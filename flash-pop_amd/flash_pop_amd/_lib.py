@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_size_t, c_void_p, POINTER, c_double
+from ctypes import c_char_p, c_int, c_longlong, c_size_t, c_void_p, POINTER, c_double
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libflashpop_hip.so"
@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
 _P, _I, _Z = c_void_p, c_int, c_size_t
 _D = POINTER(c_double)
+_L, _F = c_longlong, c_double
 
 # name -> argument types, in the order of include/flashpop_hip.h
 SIGNATURES = {
@@ -24,6 +25,9 @@ SIGNATURES = {
     "fp_pop_fused_fwd": [_P] * 7 + [_D] + [_P] * 3 + [_I] * 7 + [_P],
     "fp_pop_fused_bwd": [_P] * 7 + [_D] + [_P] * 10 + [_I] * 7 + [_P],
     "fp_retention_decode_step": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _P],
+    "fp_rotary_qk": [_P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
+    "fp_gated_group_norm_fwd": [_P, _P, _P, _L, _I, _I, _F, _P],
+    "fp_gated_group_norm_bwd": [_P, _P, _P, _P, _P, _L, _I, _I, _F, _P],
     "fp_last_error": [],
     "fp_version": [],
 }

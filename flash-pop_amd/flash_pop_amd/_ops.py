@@ -179,3 +179,78 @@ def decode_step(q, k, v, s, decays, in_place=False):
                                           _ptr(s_out), B, H, dk, dv, _stream())
     _lib.check(lib, rc)
     return o, s_out
+
+
+def _check_bf16_cuda(**tensors):
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}: flash_pop_amd runs on the GPU only")
+        assert t.dtype == torch.bfloat16, f"{name}: only bfloat16 is supported, got {t.dtype}"
+
+
+def rotary_qk(q, k, theta, start, inverse=False):
+    """q, k [B,T,H,d] (k may be None) rotated by position * theta; start an int or an int64 tensor [B]."""
+    lib = _lib.load()
+    _check_bf16_cuda(q=q, k=k)
+    if q.dim() != 4 or (k is not None and k.shape != q.shape):
+        raise ValueError(f"expected q, k [B,T,H,d]; got {tuple(q.shape)}, {None if k is None else tuple(k.shape)}")
+    B, T, H, d = q.shape
+    if tuple(theta.shape) != (d // 2,) or theta.dtype != torch.float32 or theta.device != q.device:
+        raise ValueError(f"theta must be {d // 2} floats on {q.device}")
+    start0 = 0
+    if isinstance(start, torch.Tensor):
+        if start.dim() != 1 or start.shape[0] != B:
+            raise ValueError(f"start positions: expected one per sequence ({B}), got shape {tuple(start.shape)}")
+        start = start.to(device=q.device, dtype=torch.long).contiguous()
+    else:
+        start0, start = int(start), None
+    q = q.contiguous()
+    k = None if k is None else k.contiguous()
+    q_out = torch.empty_like(q)
+    k_out = None if k is None else torch.empty_like(k)
+    if q.numel() == 0:
+        return q_out, k_out
+    with torch.cuda.device(q.device):
+        rc = lib.fp_rotary_qk(_ptr(q), _ptr(k), _ptr(q_out), _ptr(k_out), _ptr(theta.contiguous()), _ptr(start), start0,
+                              B, T, H, d, int(bool(inverse)), _stream())
+    _lib.check(lib, rc)
+    return q_out, k_out
+
+
+def _norm_shapes(r, g):
+    if r.dim() < 2 or g.numel() != r.numel() or g.shape[-1] != r.shape[-2] * r.shape[-1]:
+        raise ValueError(f"expected r [..., H, dv] and g [..., H * dv]; got {tuple(r.shape)}, {tuple(g.shape)}")
+    H, dv = r.shape[-2:]
+    return r.numel() // (H * dv), H, dv
+
+
+def gated_norm_fwd(r, g, eps):
+    """bf16(GroupNorm per head of r) * bf16(swish(g)): r [..., H, dv], g [..., H*dv] -> [..., H*dv]."""
+    lib = _lib.load()
+    _check_bf16_cuda(r=r, g=g)
+    rows, H, dv = _norm_shapes(r, g)
+    r, g = r.contiguous(), g.contiguous()
+    out = torch.empty_like(g)
+    if rows == 0:
+        return out
+    with torch.cuda.device(r.device):
+        rc = lib.fp_gated_group_norm_fwd(_ptr(r), _ptr(g), _ptr(out), rows, H, dv, float(eps), _stream())
+    _lib.check(lib, rc)
+    return out
+
+
+def gated_norm_bwd(r, g, d_out, eps):
+    lib = _lib.load()
+    _check_bf16_cuda(r=r, g=g, d_out=d_out)
+    rows, H, dv = _norm_shapes(r, g)
+    d_out = d_out.contiguous()
+    d_r, d_g = torch.empty_like(r), torch.empty_like(g)
+    if rows == 0:
+        return d_r, d_g
+    with torch.cuda.device(r.device):
+        rc = lib.fp_gated_group_norm_bwd(_ptr(r), _ptr(g), _ptr(d_out), _ptr(d_r), _ptr(d_g), rows, H, dv, float(eps),
+                                         _stream())
+    _lib.check(lib, rc)
+    return d_r, d_g

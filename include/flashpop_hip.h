@@ -122,6 +122,31 @@ int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0
 int fp_retention_decode_step(const void* q, const void* k, const void* v, const void* s_in, const double* head_decays,
                              void* o, void* s_out, int B, int H, int dk, int dv, void* stream);
 
+/* Rotary position embedding of q and k in one launch; replaces the elementwise chain of
+ * XPos.__call__ / _theta_shift (flash_pop/xpos_emb.py:32-40, 120-126), which the layer applies
+ * to q and k right before the retention op (flash_pop/retnet.py:273-278):
+ *   out[2i]   = x[2i] cos(a_i) - x[2i+1] sin(a_i),   out[2i+1] = x[2i+1] cos(a_i) + x[2i] sin(a_i)
+ *   a_i = float(position) * theta[i],  position of token t of sequence b = (start ? start[b] : start0) + t
+ *   q, k [B,T,H,d] bf16 (k_in and k_out may both be NULL); out may alias in; d a multiple of 8
+ *   theta  DEVICE, d/2 floats (the reference's 1 / 10000^linspace(0,1,d/2), xpos_emb.py:26-28)
+ *   start  DEVICE, B int64 start positions (the reference's LongTensor start_idx, xpos_emb.py:57-63), or NULL
+ *   inverse != 0 rotates by -a_i: the gradient of the op with respect to its input. */
+int fp_rotary_qk(const void* q_in, const void* k_in, void* q_out, void* k_out, const float* theta, const long long* start,
+                 long long start0, int B, int T, int H, int d, int inverse, void* stream);
+
+/* GroupNorm over each head of the retention output, then the swish gate, in one pass; replaces
+ * group_norm(retention.float()).to(dtype) * activation(g_proj(x)) in
+ * MultiScaleRetention._retention_chunkwise (flash_pop/retnet.py:294-309; GroupNorm with one group
+ * per head, no affine parameters, retnet.py:194-201; swish, retnet.py:29-30), same rounding points:
+ *   n = bf16((r - mean_h) / sqrt(var_h + eps)),  out = bf16(n * bf16(g / (1 + exp(-g))))
+ *   r [rows,H,dv] retention output, g [rows,H*dv] gate pre-activation, out [rows,H*dv]; bf16,
+ *   16-byte aligned; statistics in fp32, biased variance; dv = 8 * 2^k <= 512.
+ * The backward entry point returns d_r and d_g for a given d_out (all three shaped like r). */
+int fp_gated_group_norm_fwd(const void* r, const void* g, void* out, long long rows, int H, int dv, double eps,
+                            void* stream);
+int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, void* d_r, void* d_g, long long rows, int H,
+                            int dv, double eps, void* stream);
+
 /* Message for the last nonzero return on this thread ("" if none). */
 const char* fp_last_error(void);
 

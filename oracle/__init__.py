@@ -12,3 +12,4 @@ from .retention_oracle import (  # noqa: F401
     pop_fused_retention,
     rms_error_ratio,
 )
+from .layer_oracle import position_thetas, rotary, gated_group_norm  # noqa: F401

@@ -87,6 +87,26 @@ int decode(int B, int H, int dk, int dv) {
   return done(rc, "decode", B, 1, H, dk, dv, 0);
 }
 
+int rotary(int B, int T, int H, int d, bool per_sequence) {
+  const size_t n = (size_t)B * T * H * d;
+  uint16_t *q = buf(n), *k = buf(n), *qo = buf(n, false), *ko = buf(n, false);
+  std::vector<float> theta(d / 2);
+  for (int i = 0; i < d / 2; ++i) theta[i] = 1.0f / (float)(i + 1);
+  std::vector<long long> start(B);
+  for (int b = 0; b < B; ++b) start[b] = 100 * b;
+  int rc = fp_rotary_qk(q, k, qo, ko, theta.data(), per_sequence ? start.data() : nullptr, 7, B, T, H, d, 0, nullptr);
+  if (!rc) rc = fp_rotary_qk(qo, nullptr, qo, nullptr, theta.data(), nullptr, 7, B, T, H, d, 1, nullptr);   // q only, in place
+  return done(rc, "rotary", B, T, H, d, d, per_sequence);
+}
+
+int gated_norm(int rows, int H, int dv) {
+  const size_t n = (size_t)rows * H * dv;
+  uint16_t *r = buf(n), *g = buf(n), *d_out = buf(n), *out = buf(n, false), *d_r = buf(n, false), *d_g = buf(n, false);
+  int rc = fp_gated_group_norm_fwd(r, g, out, rows, H, dv, 1e-6, nullptr);
+  if (!rc) rc = fp_gated_group_norm_bwd(r, g, d_out, d_r, d_g, rows, H, dv, 1e-6, nullptr);
+  return done(rc, "gated norm", rows, 1, H, dv, dv, 0);
+}
+
 }  // namespace
 
 int main() {
@@ -105,5 +125,10 @@ int main() {
   rc |= fused(1, 3, 24, 64, 1, 128, 64);
   rc |= decode(2, 3, 64, 128);
   rc |= decode(1, 1, 256, 256);
+  rc |= rotary(3, 11, 2, 64, true);           // last workgroup partly idle
+  rc |= rotary(1, 5, 3, 8, false);
+  rc |= gated_norm(7, 3, 64);                 // heads past the end in the last workgroup
+  rc |= gated_norm(3, 1, 256);
+  rc |= gated_norm(9, 5, 8);
   return rc;
 }

@@ -20,6 +20,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 struct WaveShared {
   uint16_t A[64][8];
   uint16_t Bm[64][8];
+  float xchg[64];
   pthread_barrier_t bar;
 };
 
@@ -75,10 +76,21 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 FP_DEVICE float exp2_approx(float x) { return std::exp2(x); }
+FP_DEVICE void sincos_f32(float x, float& s, float& c) { s = std::sin(x); c = std::cos(x); }
+FP_DEVICE float exp_f32(float x) { return std::exp(x); }
+FP_DEVICE float rsqrt_f32(float x) { return 1.0f / std::sqrt(x); }
 
 FP_DEVICE void sched_fence() {}
 // lanes are independent OS threads here, so lane-to-lane exchange through LDS needs a real barrier
 FP_DEVICE void wave_sync() { pthread_barrier_wait(&g_lane.wave->bar); }
+FP_DEVICE float lane_xor(float v, int mask) {
+  const int lane = g_lane.tid & 63;
+  g_lane.wave->xchg[lane] = v;
+  wave_sync();
+  const float r = g_lane.wave->xchg[lane ^ mask];
+  wave_sync();
+  return r;
+}
 
 FP_DEVICE int dbg_flags() { return 0; }
 FP_DEVICE void prof_stamp(int, int) {}

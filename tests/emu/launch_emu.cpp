@@ -4,6 +4,7 @@
 #include "pass_dispatch.h"
 #include "segment_scan.h"
 #include "decode_step.h"
+#include "layer_ops.h"
 
 #include <thread>
 #include <vector>
@@ -97,4 +98,34 @@ int fpk_launch_decode(const fpk::DecodeArgs& a, void* /*stream*/, const char** e
     return 1;
   }
   return run_grid(fpk::DECODE_THREADS, a.B * a.H, fpk::decode_lds_bytes(a.dv), [&](char* l) { fpk::decode_step(a, l); });
+}
+
+int fpk_launch_rotary(const fpk::RotaryArgs& a, void* /*stream*/, const char** err) {
+  long long blocks = 0;
+  if (const char* why = fpk::plan_rotary(a, blocks)) {
+    *err = why;
+    return 1;
+  }
+  // no barriers and no lane exchanges inside: the lanes can run one after another on this thread
+  for (long long blk = 0; blk < blocks; ++blk) {
+    for (int t = 0; t < fpk::LAYER_THREADS; ++t) {
+      fprt::g_lane.tid = t;
+      fprt::g_lane.block = (int)blk;
+      fprt::g_lane.grid = (int)blocks;
+      fpk::rotary_qk(a);
+    }
+  }
+  return 0;
+}
+
+int fpk_launch_gated_norm(const fpk::GatedNormArgs& a, void* /*stream*/, const char** err) {
+  long long blocks = 0;
+  if (const char* why = fpk::plan_gated_norm(a, blocks)) {
+    *err = why;
+    return 1;
+  }
+  return run_grid(fpk::LAYER_THREADS, (int)blocks, 0, [&](char*) {
+    if (a.out) fpk::gated_norm_fwd(a);
+    else fpk::gated_norm_bwd(a);
+  });
 }

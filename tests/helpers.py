@@ -250,3 +250,49 @@ def raw_decode_step(lib, q, k, v, s, decays, stream=None, in_place=False):
     _check(lib, lib.fp_retention_decode_step(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o), _p(s_out), B, H, dk, dv,
                                              stream))
     return o, s_out
+
+
+def raw_rotary(lib, q, k, theta, start, inverse=False, stream=None, in_place=False):
+    """start: an int, or an int64 tensor [B] on the tensors' device."""
+    B, T, H, d = q.shape
+    q_out = q if in_place else torch.full_like(q, float("nan"))
+    k_out = None if k is None else (k if in_place else torch.full_like(k, float("nan")))
+    vec = start if isinstance(start, torch.Tensor) else None
+    _check(lib, lib.fp_rotary_qk(_p(q), _p(k), _p(q_out), _p(k_out), _p(theta), _p(vec), 0 if vec is not None else int(start),
+                                 B, T, H, d, int(inverse), stream))
+    return q_out, k_out
+
+
+def raw_gated_norm_fwd(lib, r, g, eps=1e-6, stream=None):
+    H, dv = r.shape[-2:]
+    rows = r.numel() // (H * dv)
+    out = torch.full_like(g, float("nan"))
+    _check(lib, lib.fp_gated_group_norm_fwd(_p(r), _p(g), _p(out), rows, H, dv, eps, stream))
+    return out
+
+
+def raw_gated_norm_bwd(lib, r, g, d_out, eps=1e-6, stream=None):
+    H, dv = r.shape[-2:]
+    rows = r.numel() // (H * dv)
+    d_r, d_g = torch.full_like(r, float("nan")), torch.full_like(g, float("nan"))
+    _check(lib, lib.fp_gated_group_norm_bwd(_p(r), _p(g), _p(d_out), _p(d_r), _p(d_g), rows, H, dv, eps, stream))
+    return d_r, d_g
+
+
+def oracle_gated_norm_grads(r, g, d_out, eps=1e-6):
+    """Autograd through the oracle's formula in fp32 on the bf16 inputs, with the forward's rounding of
+    the normalised values and of the gate kept as straight-through steps (what differentiating the
+    reference's bf16 graph gives)."""
+    import oracle
+    rf, gf = r.float().requires_grad_(True), g.float().requires_grad_(True)
+    mean = rf.mean(-1, keepdim=True)
+    var = ((rf - mean) ** 2).mean(-1, keepdim=True)
+    n = ((rf - mean) / torch.sqrt(var + eps)).flatten(-2)
+    n = n + (n.to(BF16).float() - n).detach()
+    gate = gf * torch.sigmoid(gf)
+    gate = gate + (gate.to(BF16).float() - gate).detach()
+    out = n * gate
+    check = oracle.gated_group_norm(r, g, eps).float()
+    assert float((out.detach() - check).abs().max()) <= float(check.abs().max()) * 2 ** -7
+    out.backward(d_out.float())
+    return rf.grad, gf.grad

@@ -9,8 +9,9 @@ projection, swish FFN.  Unlike the reference, d_model need not equal H * dv: v a
 projected d_model -> H * dv and the output H * dv -> d_model, which reduces to the reference's
 layer when the two are equal.
 
-The retention itself comes from a backend object, so that the same seeded model can run on the
-HIP ops and on the CPU oracle's formulas (evaluated on whatever device the tensors are on).
+The retention, the rotary embedding of q and k and the normalisation + gate come from a backend
+object, so that the same seeded model can run on the HIP ops and on plain fp32 torch formulas
+(the oracle's for the retention; evaluated on whatever device the tensors are on).
 """
 from __future__ import annotations
 
@@ -45,6 +46,12 @@ class HipBackend:
     """The ops of flash_pop_amd."""
     name = "hip"
 
+    def __init__(self, layer_ops: bool = True):
+        """layer_ops=False keeps the rotary embedding and the normalisation + gate as eager torch
+        formulas around the HIP retention ops (what a caller that only switches the ops gets)."""
+        self._xpos = {}
+        self.layer_ops = layer_ops
+
     def plain(self, q, k, v, s, decays):
         from flash_pop_amd import fused_chunk_retention
         return fused_chunk_retention(q, k, v, s, decays)
@@ -56,6 +63,21 @@ class HipBackend:
     def step(self, q, k, v, s, decays, in_place=False):
         from flash_pop_amd import retention_recurrent
         return retention_recurrent(q, k, v, decays, s, in_place=in_place)
+
+    def rotate(self, q, k, start):
+        if not self.layer_ops:
+            return OracleBackend.rotate(self, q, k, start)
+        from flash_pop_amd import XPos
+        d = q.shape[-1]
+        if d not in self._xpos:
+            self._xpos[d] = XPos(d)
+        return self._xpos[d](q, k, start)
+
+    def norm_gate(self, retention, gate):
+        if not self.layer_ops:
+            return OracleBackend.norm_gate(self, retention, gate)
+        from flash_pop_amd import gated_group_norm
+        return gated_group_norm(retention, gate, 1e-6)
 
 
 class OracleBackend:
@@ -73,18 +95,29 @@ class OracleBackend:
         o, o_s, last = oracle.pop_fused_retention(f(q), f(k), f(v), f(s), f(q_s), f(k_s), f(v_s), decays, block)
         return o.to(q.dtype), o_s.to(q.dtype), last.to(q.dtype)
 
+    def rotate(self, q, k, start):
+        return rotate(q, start), rotate(k, start)
+
+    def norm_gate(self, retention, gate):
+        r = retention.float()
+        r = (r - r.mean(-1, keepdim=True)) * torch.rsqrt(r.var(-1, unbiased=False, keepdim=True) + 1e-6)
+        return r.flatten(-2).to(gate.dtype) * F.silu(gate)
+
     def step(self, q, k, v, s, decays, in_place=False):
         import oracle
         o, S = oracle.recurrent_step(q.float(), k.float(), v.float(), None if s is None else s.float(), decays)
         return o.to(q.dtype), S.to(q.dtype)
 
 
-def rotate(x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+def rotate(x: torch.Tensor, start) -> torch.Tensor:
     """Pairs (x[2i], x[2i+1]) rotated by position * theta_i, theta_i = 10000^(-i / (d/2 - 1))
-    (flash_pop/xpos_emb.py:24-40).  x [..., n, h, d]; positions broadcastable to [..., n]."""
-    d = x.shape[-1]
-    theta = 1.0 / (10000.0 ** torch.linspace(0, 1, d // 2, device=x.device))
-    ang = positions[..., None, None].float() * theta                     # [..., n, 1, d/2]
+    (flash_pop/xpos_emb.py:24-40).  x [B, T, H, d]; the position of token t of sequence b is
+    start + t (start an int) or start[b] + t (start an integer tensor of B elements)."""
+    d, T = x.shape[-1], x.shape[1]
+    theta = 1.0 / (10000.0 ** torch.linspace(0, 1, d // 2)).to(x.device)
+    first = start.reshape(-1, 1) if isinstance(start, torch.Tensor) else start
+    positions = first + torch.arange(T, device=x.device)[None]              # [B or 1, T]
+    ang = positions[..., None, None].float() * theta                       # [B or 1, T, 1, d/2]
     sin, cos = torch.sin(ang), torch.cos(ang)
     xf = x.float()
     even, odd = xf[..., 0::2], xf[..., 1::2]
@@ -107,20 +140,16 @@ class Retention(nn.Module):
             nn.init.zeros_(lin.bias)
         self.decays = head_decays(H)
 
-    def qkv(self, x, positions):
+    def qkv(self, backend, x, start):
+        """x [B, T, D]; start: position of the first token, an int or one integer per sequence."""
         H, dk, dv = self.cfg.heads, self.cfg.dk, self.cfg.dv
-        q = rotate(self.q_proj(x).unflatten(-1, (H, dk)), positions)
-        k = rotate(self.k_proj(x).unflatten(-1, (H, dk)), positions)
+        q, k = backend.rotate(self.q_proj(x).unflatten(-1, (H, dk)), self.k_proj(x).unflatten(-1, (H, dk)), start)
         v = self.v_proj(x).unflatten(-1, (H, dv))
         return q, k, v
 
-    def finish(self, x, retention):
-        """GroupNorm per head in fp32, gate, output projection.  retention [..., H, dv]."""
-        H = self.cfg.heads
-        r = retention.float()
-        r = (r - r.mean(-1, keepdim=True)) * torch.rsqrt(r.var(-1, unbiased=False, keepdim=True) + 1e-6)
-        r = r.flatten(-2).to(x.dtype)
-        return self.out_proj(r * F.silu(self.g_proj(x)))
+    def finish(self, backend, x, retention):
+        """GroupNorm per head in fp32, swish gate, output projection.  retention [..., H, dv]."""
+        return self.out_proj(backend.norm_gate(retention, self.g_proj(x)))
 
 
 class Layer(nn.Module):
@@ -149,32 +178,30 @@ class Layer(nn.Module):
         B, T = x.shape[:2]
         n1 = sfx.shape[0] // B
         xn, sn = self._norm(self.norm1, x), self._norm(self.norm1, sfx)
-        pos = start + torch.arange(T, device=x.device)
         sfx_start = (start + torch.arange(n1, device=x.device) * cfg.block).repeat(B)       # pop_retnet.py:175-179
-        spos = sfx_start[:, None] + torch.arange(sfx.shape[1], device=x.device)[None]
-        q, k, v = r.qkv(xn, pos)
-        qs, ks, vs = r.qkv(sn, spos)
+        q, k, v = r.qkv(backend, xn, start)
+        qs, ks, vs = r.qkv(backend, sn, sfx_start)
         o, o_s, last = backend.pop(q, k, v, state, r.decays, cfg.block, qs, ks, vs)
-        x = self._ffn(x + r.finish(xn, o))
-        sfx = self._ffn(sfx + r.finish(sn, o_s))
+        x = self._ffn(x + r.finish(backend, xn, o))
+        sfx = self._ffn(sfx + r.finish(backend, sn, o_s))
         return x, sfx, last
 
     def chunkwise(self, backend, x, start, state):
         r = self.retention
         xn = self._norm(self.norm1, x)
-        q, k, v = r.qkv(xn, start + torch.arange(x.shape[1], device=x.device))
+        q, k, v = r.qkv(backend, xn, start)
         o, state = backend.plain(q, k, v, state, r.decays)
-        return self._ffn(x + r.finish(xn, o)), state
+        return self._ffn(x + r.finish(backend, xn, o)), state
 
     def recurrent(self, backend, x, index, state, in_place=False):
         """x [B, D], one token at position `index` (an int, or a one-element tensor on the device)
         (flash_pop/retnet.py:325-366, 493-512)."""
         r = self.retention
         xn = self._norm(self.norm1, x)
-        pos = index if isinstance(index, torch.Tensor) else torch.full((1,), index, device=x.device)
-        q, k, v = r.qkv(xn[:, None], pos)
+        start = index.expand(x.shape[0]) if isinstance(index, torch.Tensor) else index
+        q, k, v = r.qkv(backend, xn[:, None], start)
         o, state = backend.step(q[:, 0], k[:, 0], v[:, 0], state, r.decays, in_place=in_place)
-        return self._ffn(x + r.finish(xn, o)), state
+        return self._ffn(x + r.finish(backend, xn, o)), state
 
 
 class PopRetNetLM(nn.Module):

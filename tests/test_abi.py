@@ -31,7 +31,7 @@ def test_header_and_binding_agree(lib):
     assert names == sorted(_lib.SIGNATURES), (names, sorted(_lib.SIGNATURES))
     for n in names:
         assert hasattr(lib, n), f"{n} not exported"
-    assert lib.fp_version() == 1003
+    assert lib.fp_version() == 1004
 
 
 def test_argument_checks_return_codes(lib):
@@ -108,3 +108,37 @@ def test_new_python_wrappers_refuse_cpu_tensors():
         retention_recurrent(x, x, x, (0.9, 0.9), None)
     with pytest.raises(ValueError, match=r"\[B,H,dk\]"):
         retention_recurrent(x[0], x[0], x[0], (0.9, 0.9), None)
+
+
+def test_layer_entry_points_check_their_arguments(lib):
+    p, odd, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1008), None
+    # rotary: NULLs, k given on one side only, shape, head dimension, alignment
+    assert lib.fp_rotary_qk(null, p, p, p, p, null, 0, 1, 4, 2, 64, 0, None) == -1
+    assert lib.fp_rotary_qk(p, p, p, p, null, null, 0, 1, 4, 2, 64, 0, None) == -1
+    assert lib.fp_rotary_qk(p, p, p, null, p, null, 0, 1, 4, 2, 64, 0, None) == -1
+    assert lib.fp_rotary_qk(p, p, p, p, p, null, 0, 1, 0, 2, 64, 0, None) == -2
+    assert lib.fp_rotary_qk(p, p, p, p, p, null, 0, 1, 4, 2, 60, 0, None) == -3
+    assert lib.fp_rotary_qk(odd, p, p, p, p, null, 0, 1, 4, 2, 64, 0, None) == -2
+    assert b"aligned" in lib.fp_last_error()
+    # gated norm: NULLs, rows, group width (8 * 2^k <= 512), eps, alignment
+    assert lib.fp_gated_group_norm_fwd(p, null, p, 4, 2, 64, 1e-6, None) == -1
+    assert lib.fp_gated_group_norm_bwd(p, p, p, p, null, 4, 2, 64, 1e-6, None) == -1
+    assert lib.fp_gated_group_norm_fwd(p, p, p, 0, 2, 64, 1e-6, None) == -2
+    assert lib.fp_gated_group_norm_fwd(p, p, p, 4, 2, 96, 1e-6, None) == -3
+    assert lib.fp_gated_group_norm_fwd(p, p, p, 4, 2, 1024, 1e-6, None) == -3
+    assert lib.fp_gated_group_norm_fwd(p, p, p, 4, 2, 64, -1.0, None) == -2
+    assert lib.fp_gated_group_norm_bwd(p, p, odd, p, p, 4, 2, 64, 1e-6, None) == -2
+
+
+def test_layer_wrappers_refuse_cpu_tensors_and_bad_shapes():
+    import torch
+    from flash_pop_amd import XPos, gated_group_norm
+    q = torch.zeros(2, 8, 2, 64, dtype=torch.bfloat16)
+    xpos = XPos(64)
+    assert xpos.thetas.shape == (32,) and float(xpos.thetas[0]) == 1.0
+    with pytest.raises(RuntimeError, match="GPU only"):
+        xpos(q, q, 0)
+    with pytest.raises(AssertionError, match="head dimension"):
+        XPos(128)(q, q, 0)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        gated_group_norm(q, q.flatten(-2))

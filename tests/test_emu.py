@@ -143,3 +143,41 @@ def test_gamma_one_and_tiny(emu_lib):
     o_ref, S_ref = hp.oracle_plain(q, k, v, s, decays)
     hp.assert_close(o, o_ref, "o")
     hp.assert_close(S, S_ref, "S")
+
+
+@pytest.mark.parametrize("B,T,H,d,vec", [(2, 37, 3, 64, False), (3, 5, 2, 128, True), (1, 300, 1, 8, False)])
+def test_rotary(emu_lib, B, T, H, d, vec):
+    """Rotation of q and k (also q alone, in place, and back) against the oracle."""
+    g = torch.Generator().manual_seed(d + T)
+    q, k = (torch.randn(B, T, H, d, generator=g).to(hp.BF16) for _ in range(2))
+    theta = oracle.position_thetas(d)
+    start = torch.tensor([7, 4000, 123456][:B]) if vec else 1000
+    pos = (start[:, None] if vec else start) + torch.arange(T)[None]
+    rq, rk = hp.raw_rotary(emu_lib, q, k, theta, start)
+    assert torch.equal(rq, oracle.rotary(q, pos, theta)) and torch.equal(rk, oracle.rotary(k, pos, theta))
+    only_q, none = hp.raw_rotary(emu_lib, q, None, theta, start)
+    assert none is None and torch.equal(only_q, rq)
+    back_q, back_k = hp.raw_rotary(emu_lib, rq, rk, theta, start, inverse=True)
+    assert torch.equal(back_q, oracle.rotary(rq, pos, theta, inverse=True))
+    hp.assert_close(back_k, k.float(), "round trip")
+    q2, k2 = q.clone(), k.clone()
+    hp.raw_rotary(emu_lib, q2, k2, theta, start, in_place=True)
+    assert torch.equal(q2, rq) and torch.equal(k2, rk)
+
+
+@pytest.mark.parametrize("rows,H,dv", [(19, 3, 64), (5, 2, 128), (3, 1, 256), (70, 5, 8)])
+def test_gated_group_norm(emu_lib, rows, H, dv):
+    g = torch.Generator().manual_seed(rows + dv)
+    r = (torch.randn(rows, H, dv, generator=g) * 2 + 0.5).to(hp.BF16)
+    gate = torch.randn(rows, H * dv, generator=g).to(hp.BF16)
+    d_out = torch.randn(rows, H * dv, generator=g).to(hp.BF16)
+    out = hp.raw_gated_norm_fwd(emu_lib, r, gate)
+    ref = oracle.gated_group_norm(r, gate)
+    # same rounding points as the oracle: equal except where an fp32 value sits on a bf16 rounding boundary
+    differ = (out.float() - ref.float()).abs()
+    assert float((differ > 0).float().mean()) < 0.01, float((differ > 0).float().mean())
+    hp.assert_close(out, ref.float(), "out")
+    d_r, d_g = hp.raw_gated_norm_bwd(emu_lib, r, gate, d_out)
+    d_r_ref, d_g_ref = hp.oracle_gated_norm_grads(r, gate, d_out)
+    hp.assert_close(d_r, d_r_ref, "d_r")
+    hp.assert_close(d_g, d_g_ref, "d_g")
