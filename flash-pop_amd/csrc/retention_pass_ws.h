@@ -5,12 +5,16 @@
 // Z / Y / R.  Hardware places waves w and w + 4 on the same SIMD, so every SIMD runs one
 // wave of each role:
 //
-//   readout waves (0..3)  scores^T = W X^T -> P (bf16, in registers) ; Y^T = wread (R X^T) + Z^T P^T
-//                         -> Y tile into LDS.  2 x 2 grid: `ib` = 32 chunk rows, `nb` = 32 columns.
-//                         A wave's rows meet two 32 x 32 score tiles: the diagonal one, whose
+//   readout waves (0..3)  scores^T = W X^T -> P (bf16) ; Y^T = wread (R X^T) + Z^T P^T -> Y tile
+//                         into LDS.  2 x 2 grid: `ib` = 32 chunk rows, `nb` = 32 columns.  The
+//                         rows of a block meet two 32 x 32 score tiles: the diagonal one, whose
 //                         masked half is cleared after conversion, and one that lies wholly inside
-//                         or wholly outside the decay window.  The loop has no data-dependent
-//                         branches; it exists in two copies, with and without the second tile.
+//                         or wholly outside the decay window.  Every live tile is computed once,
+//                         the diagonal one by the wave with nb = 0 and the other one by the wave
+//                         with nb = 1, and handed to the partner wave of the row block through a
+//                         2 KB LDS tile in operand layout (a barrier in the middle of the item).
+//                         The loop has no data-dependent branches; it exists in three copies (two
+//                         live tiles; one, made here; one, made by the partner).
 //                         They also feed X and Z: bounds-checked buffer loads into registers, X
 //                         copied and Z transposed into LDS one chunk ahead, and they store the Y
 //                         tile of the previous chunk.
@@ -24,8 +28,9 @@
 //
 // LDS tiles are double-buffered: while the readout waves work on chunk i from stage i & 1 the
 // state waves finish chunk i's state update and fill stage (i + 1) & 1 with chunk i + 1.  One
-// workgroup barrier per chunk.  The weighted, transposed W tile is private to the state wave
-// that both writes and reads it, so it needs no second buffer and no barrier.
+// workgroup barrier ends a chunk and one in its middle publishes the P tiles.  The weighted,
+// transposed W tile is private to the state wave that both writes and reads it, so it needs no
+// second buffer and no barrier.
 //
 // Within a chunk the code is laid out in phases separated by scheduling fences: all LDS
 // operands of a phase are requested first, the MFMAs that consume them follow back to back,
@@ -43,7 +48,8 @@ constexpr int lds_bytes_ws(int dA) {
               + 2 * BV * (CH + 4)      // Z transposed, two stages
               + 2 * BV * (dA + 8)      // bf16 copy of R (transposed), two stages
               + 2 * CH * (BV + 8)      // Y staging, two stages
-              + 4 * 32 * (CH + 4));    // weighted W transposed, one 32-row slab per state wave
+              + 4 * 32 * (CH + 4)      // weighted W transposed, one 32-row slab per state wave
+              + 3 * 32 * 32);          // P tiles handed between the readout waves of a row block
 }
 
 template <int H>
@@ -98,6 +104,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   uint16_t* const RT = ZT + 2 * BV * T_LD;
   uint16_t* const YB = RT + 2 * BV * RT_LD;
   uint16_t* const WT = YB + 2 * CH * YB_LD;
+  uint16_t* const PB = WT + 4 * 32 * T_LD;   // [diagonal tile of row block 0, of row block 1, the other tile][k-step][lane]
 
   const int tid = fprt::thread_index();
   const int wave = tid >> 6, lane = tid & 63;
@@ -218,33 +225,39 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   if (!state_role) {
     // =============================== readout waves ===============================
     const int ib = wave >> 1, nb = wave & 1;
-    // Of the two 32-token score tiles of this wave's rows, the "diagonal" one (tokens 32 ib ..)
-    // is half masked; the "other" one (tokens 32 (1 - ib) ..) lies either wholly inside the
-    // decay window or wholly outside it.  Masked scores are zeroed by clearing their bits after
-    // the bf16 conversion, so that inf or nan in a masked operand cannot leak through 0 * x.
+    // The rows of block `ib` meet two 32-token score tiles: the "diagonal" one (tokens 32 ib ..),
+    // half masked, and the "other" one (tokens 32 (1 - ib) ..), which lies either wholly inside
+    // the decay window or wholly outside it.  Each live tile is computed once: the diagonal one
+    // by the wave with nb = 0, the other one by the wave with nb = 1, and handed to the partner
+    // wave of the row block through LDS (the accumulator layout of scores^T is, lane for lane,
+    // the operand layout of the next product in both waves).  Masked scores are zeroed by
+    // clearing their bits after the bf16 conversion, so that inf or nan in a masked operand
+    // cannot leak through 0 * x.
     const bool other_live = rev ? (ib == 0) : (ib == 1);
-    float mw_d[16], mw_o[16];
-    uint32_t keep_d[8];
+    const bool makes_diag = nb == 0;
+    float mw[16];          // decay weights of the tile this wave computes
+    uint32_t keep[8];      // bits to keep after conversion (all of them off the diagonal)
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int jl = acc_row(r, g);
       const int d = rev ? (jl - c) : (c - jl);          // distance inside the diagonal tile
-      mw_d[r] = p.s_intra * fprt::exp2_approx((float)(d >= 0 ? d : 0) * lg);
-      mw_o[r] = p.s_intra * fprt::exp2_approx((float)(32 + d) * lg);
+      mw[r] = p.s_intra * fprt::exp2_approx((float)(makes_diag ? (d >= 0 ? d : 0) : 32 + d) * lg);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int d0 = rev ? (acc_row(2 * e, g) - c) : (c - acc_row(2 * e, g));
       const int d1 = rev ? (acc_row(2 * e + 1, g) - c) : (c - acc_row(2 * e + 1, g));
-      keep_d[e] = (d0 >= 0 ? 0x0000ffffu : 0u) | (d1 >= 0 ? 0xffff0000u : 0u);
+      keep[e] = makes_diag ? ((d0 >= 0 ? 0x0000ffffu : 0u) | (d1 >= 0 ? 0xffff0000u : 0u)) : 0xffffffffu;
     }
     const int i_row = 32 * ib + c;                 // this lane's chunk row (query index)
     const int x_off = i_row * X_LD + 8 * g;
-    const int wd_off = (32 * ib + c) * X_LD + 8 * g;
-    const int wo_off = (32 * (1 - ib) + c) * X_LD + 8 * g;
+    const int w_off = (32 * (makes_diag ? ib : 1 - ib) + c) * X_LD + 8 * g;   // W rows of this wave's score tile
+    uint16_t* const p_mine = PB + (makes_diag ? ib : 2) * 1024 + lane * 8;      // + 512 per k-step
+    const uint16_t* const p_theirs = PB + (makes_diag ? 2 : ib) * 1024 + lane * 8;
     const int r_off = (32 * nb + c) * RT_LD + 8 * g;
-    const int zd_off = (32 * nb + c) * T_LD + 4 * g + 32 * ib;
-    const int zo_off = (32 * nb + c) * T_LD + 4 * g + 32 * (1 - ib);
+    // Z^T fragments: the tokens of the tile this wave makes, and of the tile it is handed
+    const int zm_off = (32 * nb + c) * T_LD + 4 * g + 32 * (makes_diag ? ib : 1 - ib);
+    const int zh_off = (32 * nb + c) * T_LD + 4 * g + 32 * (makes_diag ? 1 - ib : ib);
     const int y_off = i_row * YB_LD + 32 * nb + 4 * g;
     const float wread_fwd = p.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
 
@@ -337,10 +350,11 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     // reloaded with item it + 2.  Returns false after the last item.  `half` is the parity of `it`
     // as a type: with NH = 2 the first visit of a chunk opens the accumulators and the second
     // closes them; with NH = 1 every visit does both.
-    f32x16 yacc, sd, so;
-    auto iteration = [&](auto half, auto with_other, int it) -> bool {
+    f32x16 yacc, sc;
+    // `makes`: this wave computes a score tile.  `both`: the rows of this wave see two live tiles.
+    auto iteration = [&](auto half, auto makes_c, auto both_c, int it) -> bool {
       constexpr int HF = decltype(half)::value;
-      constexpr bool OTHER = decltype(with_other)::value;   // false: the other tile is outside the decay window
+      constexpr bool MAKES = decltype(makes_c)::value, BOTH = decltype(both_c)::value;
       constexpr bool opens = NH == 1 || HF == 0, closes = NH == 1 || HF == 1;
       const int s = it & 1;
       const int L = ck.L;
@@ -371,21 +385,24 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         return ck.ok;
       }
       if (dbg & 2) {
+        if (closes) fprt::block_sync();
         fprt::block_sync();
         ckp = ck;
         ck = ck1;
         ck1 = ck2;
         return ck.ok;
       }
-      // ---- phase 0: request X, R and the diagonal W tile
-      u32x4 xf[KS], rf[KS], wd[KS], wo[KS], zd[2], zo[2];
+      // ---- phase 0: request X, R and the W rows of this wave's score tile
+      u32x4 xf[KS], rf[KS], wf[KS], zm[2], zh[2];
 #pragma unroll
       for (int t = 0; t < KS; ++t) {
         xf[t] = ld128(xs + x_off + 16 * t);
         rf[t] = ld128(rt + r_off + 16 * t);
       }
+      if (MAKES) {
 #pragma unroll
-      for (int t = 0; t < KS; ++t) wd[t] = ld128(ws + wd_off + 16 * t);
+        for (int t = 0; t < KS; ++t) wf[t] = ld128(ws + w_off + 16 * t);
+      }
       fprt::sched_fence();
 
       // ---- phase 1: read-out of the carried state, Y^T[n][i] = sum_a R[a][n] X[i][a]
@@ -395,46 +412,42 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       fprt::sched_fence();
       fprt::prof_stamp(it, 1);
 
-      // ---- phase 2: scores^T of the diagonal tile; the other W tile and Z arrive meanwhile (the
-      // W tile takes over the registers of the R fragments); X of chunk it + 1 goes to the other stage
-      if (OTHER) {
-#pragma unroll
-        for (int t = 0; t < KS; ++t) wo[t] = ld128(ws + wo_off + 16 * t);
-      }
+      // ---- phase 2: scores^T of this wave's tile; Z arrives meanwhile; X of chunk it + 1 goes
+      // to the other stage
       if (closes) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          zd[t] = ld_token_frag(zt + zd_off + 16 * t);
-          if (OTHER) zo[t] = ld_token_frag(zt + zo_off + 16 * t);
+          if (MAKES) zm[t] = ld_token_frag(zt + zm_off + 16 * t);
+          if (BOTH || !MAKES) zh[t] = ld_token_frag(zt + zh_off + 16 * t);
         }
       }
-      if (opens) sd = f32x16{0};
+      if (MAKES) {
+        if (opens) sc = f32x16{0};
 #pragma unroll
-      for (int t = 0; t < KS; ++t) sd = fprt::mfma_32x32x16_bf16(wd[t], xf[t], sd);
+        for (int t = 0; t < KS; ++t) sc = fprt::mfma_32x32x16_bf16(wf[t], xf[t], sc);
+      }
       feed_store_x(feed, s ^ 1);
       feed_load_x(feed, ck2);
       fprt::sched_fence();
       fprt::prof_stamp(it, 2);
 
-      // ---- phase 3: scores^T of the other tile; the read-out is scaled and P of the diagonal
-      // tile converted in its shadow, and Z of chunk it + 1 is transposed into the other stage.
-      // Accumulator element r = 8 t + e is token 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the
-      // order the Z fragments are read in.
-      if (opens) so = f32x16{0};
-      if (OTHER) {
-#pragma unroll
-        for (int t = 0; t < KS; ++t) so = fprt::mfma_32x32x16_bf16(wo[t], xf[t], so);
-      }
-      u32x4 pd[2], po[2];
+      // ---- phase 3: the read-out is scaled, P converted and put where the partner wave finds
+      // it, and Z of chunk it + 1 is transposed into the other stage.  Accumulator element
+      // r = 8 t + e is token 16 t + 8 (e / 4) + 4 g + e % 4 of its tile, the order the Z
+      // fragments are read in.
+      u32x4 pm[2], pt[2];
       if (closes) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) yacc[r] *= wread;
+        if (MAKES) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+          for (int t = 0; t < 2; ++t) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = 8 * t + 2 * e;
-            pd[t][e] = fprt::pack_bf16x2(sd[r] * mw_d[r], sd[r + 1] * mw_d[r + 1]) & keep_d[4 * t + e];
+            for (int e = 0; e < 4; ++e) {
+              const int r = 8 * t + 2 * e;
+              pm[t][e] = fprt::pack_bf16x2(sc[r] * mw[r], sc[r + 1] * mw[r + 1]) & keep[4 * t + e];
+            }
+            st128(p_mine + 512 * t, pm[t]);
           }
         }
       }
@@ -449,21 +462,22 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
         ck1 = ck2;
         return true;
       }
+      fprt::block_sync();   // every P tile of this chunk is in LDS
 
-      // ---- phase 4: Y^T += Z^T P^T
+      // ---- phase 4: Y^T += Z^T P^T with the own tile from registers and the partner's from LDS.
+      // A wave that made the diagonal tile gets the other one, and the other way round; a wave
+      // that made nothing gets the diagonal one.
+      if (BOTH || !MAKES) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zd[t], pd[t], yacc);
-      if (OTHER) {
+        for (int t = 0; t < 2; ++t) pt[t] = ld128(p_theirs + 512 * t);
+      }
+      if (MAKES) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zm[t], pm[t], yacc);
+      }
+      if (BOTH || !MAKES) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = 8 * t + 2 * e;
-            po[t][e] = fprt::pack_bf16x2(so[r] * mw_o[r], so[r + 1] * mw_o[r + 1]);
-          }
-        }
-#pragma unroll
-        for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zo[t], po[t], yacc);
+        for (int t = 0; t < 2; ++t) yacc = fprt::mfma_32x32x16_bf16(zh[t], pt[t], yacc);
       }
       fprt::sched_fence();
 
@@ -485,16 +499,22 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
       if (!ck.ok) drain_y(ckp, s);   // the last Y tile
       return ck.ok;
     };
-    // Two copies of the loop, chosen once: the waves whose other tile is dead run the one without it.
+    // Three copies of the loop, chosen once per wave: two live tiles and this wave makes one of
+    // them; one live tile made by this wave; one live tile made by the partner.
     if (other_live) {
       for (int it = 0;; it += 2) {
-        if (!iteration(Half<0>{}, Half<1>{}, it)) break;
-        if (!iteration(Half<1>{}, Half<1>{}, it + 1)) break;
+        if (!iteration(Half<0>{}, Half<1>{}, Half<1>{}, it)) break;
+        if (!iteration(Half<1>{}, Half<1>{}, Half<1>{}, it + 1)) break;
+      }
+    } else if (makes_diag) {
+      for (int it = 0;; it += 2) {
+        if (!iteration(Half<0>{}, Half<1>{}, Half<0>{}, it)) break;
+        if (!iteration(Half<1>{}, Half<1>{}, Half<0>{}, it + 1)) break;
       }
     } else {
       for (int it = 0;; it += 2) {
-        if (!iteration(Half<0>{}, Half<0>{}, it)) break;
-        if (!iteration(Half<1>{}, Half<0>{}, it + 1)) break;
+        if (!iteration(Half<0>{}, Half<0>{}, Half<0>{}, it)) break;
+        if (!iteration(Half<1>{}, Half<0>{}, Half<0>{}, it + 1)) break;
       }
     }
     return;
@@ -738,6 +758,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (MULTI) tile_load(t_init, (fresh && p.R0) ? state_matrix(p.R0, nxt.b) : nullptr, fresh, 0);
 
     if (dbg & 4) {
+      if (!STATE && closes) fprt::block_sync();
       fprt::block_sync();
       if (!nxt.ok) return false;
       cur = nxt;
@@ -799,6 +820,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     store_transposed(wregs, nxt);
     fprt::sched_fence();
     fprt::prof_stamp(it, 2);
+    if (!STATE && closes) fprt::block_sync();   // the readout waves hand their P tiles to each other here
 
     // ---- phase 2: second half of the state update; the row-major copies go out in its shadow
 #pragma unroll
