@@ -11,7 +11,8 @@
 //
 // The column dimension dB is split over workgroups, the contraction dimension dA never is,
 // so no pass needs a cross-workgroup reduction.  The dq pass re-runs the state recurrence
-// instead of reading stored chunk states; the dk and dv passes each carry dS.
+// instead of reading stored chunk states; the dk and dv passes each carry dS and, when dk == dv,
+// share one launch so that the q and dO rows both of them read come from HBM once.
 //
 // The POP entry points add block states to these passes (written by fwd, their gradients read
 // by dk and dv); the fused POP entry points add the suffix tensors in the same four roles; the
@@ -87,6 +88,19 @@ int run(const fpk::PassArgs& a, void* stream, const char* what) {
   return FP_OK;
 }
 
+// The dk and dv passes read the same q and dO rows walking in the same direction.  When dk == dv
+// they are the same kernel with the same grid, and one launch runs the workgroups of a stream in
+// both passes side by side: q and dO then come from HBM once instead of twice.
+int run_dk_dv(const fpk::PassArgs& pass_dk, const fpk::PassArgs& pass_dv, void* stream, const char* what) {
+  if (pass_dk.dA != pass_dv.dA) {
+    if (int rc = run(pass_dk, stream, what)) return rc;
+    return run(pass_dv, stream, what);
+  }
+  const char* msg = "";
+  if (fpk_launch_pass_pair(pass_dk, pass_dv, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s passes: %s", what, msg);
+  return FP_OK;
+}
+
 // R = S, dk x dv, rows contiguous in dv
 void plain_state(fpk::PassArgs& a, const Shape& s) {
   a.dA = s.dk;
@@ -140,16 +154,16 @@ int backward(const Shape& s, const void* q, const void* k, const void* v, const 
   a.block = d_blocks ? block : 0; a.nblk = nblk;
   a.reverse = 1;
   a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
-  if ((rc = run(a, stream, "dk")) != FP_OK) return rc;
 
-  fill_common(a, s, decays);   // dv (+ d_s0)
-  a.X = in(k); a.W = in(q); a.Z = in(d_o); a.Y = out(dv_);
-  a.R0 = in(d_s_out); a.Bin = in(d_blocks); a.Rout = out(d_s0);
-  plain_state(a, s);
-  a.block = d_blocks ? block : 0; a.nblk = nblk;
-  a.reverse = 1;
-  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
-  return run(a, stream, "dv");
+  fpk::PassArgs b;
+  fill_common(b, s, decays);   // dv (+ d_s0)
+  b.X = in(k); b.W = in(q); b.Z = in(d_o); b.Y = out(dv_);
+  b.R0 = in(d_s_out); b.Bin = in(d_blocks); b.Rout = out(d_s0);
+  plain_state(b, s);
+  b.block = d_blocks ? block : 0; b.nblk = nblk;
+  b.reverse = 1;
+  b.s_intra = sc; b.s_read = sc; b.s_update = 1.f;
+  return run_dk_dv(a, b, stream, "dk / dv");
 }
 
 // ---- long sequences, few streams: cut every sequence into segments ---------------------------
@@ -267,15 +281,15 @@ int backward_split(const Shape& s, int segments, const void* q, const void* k, c
   transposed_state(a, seg);
   a.reverse = 1;
   a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
-  if ((rc = run(a, stream, "dk")) != FP_OK) return rc;
 
-  fill_common(a, seg, decays);
-  a.X = in(k); a.W = in(q); a.Z = in(d_o); a.Y = out(dv_);
-  a.R0 = w.start;
-  plain_state(a, seg);
-  a.reverse = 1;
-  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
-  return run(a, stream, "dv");
+  fpk::PassArgs b;
+  fill_common(b, seg, decays);
+  b.X = in(k); b.W = in(q); b.Z = in(d_o); b.Y = out(dv_);
+  b.R0 = w.start;
+  plain_state(b, seg);
+  b.reverse = 1;
+  b.s_intra = sc; b.s_read = sc; b.s_update = 1.f;
+  return run_dk_dv(a, b, stream, "dk / dv");
 }
 
 int check_workspace(const Shape& s, int segments, const void* workspace, size_t bytes) {
@@ -352,16 +366,16 @@ int fused_backward(const Shape& s, const void* q, const void* k, const void* v, 
   suffix_walk(a, s, block, x.len, x.v, d_o_sfx, x.q, dk_sfx);
   a.reverse = 1;
   a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
-  if ((rc = run(a, stream, "fused dk")) != FP_OK) return rc;
 
-  fill_common(a, s, decays);   // dv (+ d_s0)
-  a.X = in(k); a.W = in(q); a.Z = in(d_o); a.Y = out(dv_);
-  a.R0 = in(d_s_out); a.Rout = out(d_s0);
-  plain_state(a, s);
-  suffix_walk(a, s, block, x.len, x.k, x.q, d_o_sfx, dv_sfx);
-  a.reverse = 1;
-  a.s_intra = sc; a.s_read = sc; a.s_update = 1.f;
-  return run(a, stream, "fused dv");
+  fpk::PassArgs b;
+  fill_common(b, s, decays);   // dv (+ d_s0)
+  b.X = in(k); b.W = in(q); b.Z = in(d_o); b.Y = out(dv_);
+  b.R0 = in(d_s_out); b.Rout = out(d_s0);
+  plain_state(b, s);
+  suffix_walk(b, s, block, x.len, x.k, x.q, d_o_sfx, dv_sfx);
+  b.reverse = 1;
+  b.s_intra = sc; b.s_read = sc; b.s_update = 1.f;
+  return run_dk_dv(a, b, stream, "fused dk / dv");
 }
 
 }  // namespace

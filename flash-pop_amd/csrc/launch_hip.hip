@@ -13,7 +13,18 @@ namespace {
 template <int DA, int MODE, int NH = 1>
 __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(const fpk::PassArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::retention_pass_ws<DA, MODE, NH>(args, lds);
+  const int nwg = fprt::grid_size();
+  fpk::retention_pass_ws<DA, MODE, NH>(args, fpk::tensors_of(args), lds, fpk::place_workgroup(fprt::block_index(), nwg, 1).wg, nwg);
+}
+
+// Two independent passes of the same shape in one grid (see fpk_launch_pass_pair).
+template <int DA, int MODE, int NH = 1>
+__global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_pair_kernel(const fpk::PassArgs first,
+                                                                               const fpk::PassTensors second) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int nwg = fprt::grid_size() / 2;
+  const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, 2);
+  fpk::retention_pass_ws<DA, MODE, NH>(first, id.pass ? second : fpk::tensors_of(first), lds, id.wg, nwg);
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -42,12 +53,12 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(cons
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
-static_assert(fpk::PASS_KERNELS <= 32, "one bit per kernel instantiation");
+static_assert(2 * fpk::PASS_KERNELS <= 32, "one bit per kernel instantiation, single and paired");
 std::atomic<uint32_t> g_armed[kMaxDevices];
 
-template <typename Kernel>
-int launch(Kernel kernel, int threads, int lds, int slot, const fpk::PassArgs& a, hipStream_t stream,
-           const char** err) {
+template <typename Kernel, typename... Second>
+int launch(Kernel kernel, int threads, int lds, int slot, hipStream_t stream, const char** err, const fpk::PassArgs& a,
+           const Second&... more) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     *err = "hipGetDevice failed";
@@ -63,8 +74,8 @@ int launch(Kernel kernel, int threads, int lds, int slot, const fpk::PassArgs& a
     }
     if (tracked) g_armed[dev].fetch_or(1u << slot, std::memory_order_release);
   }
-  const int nwg = a.slots * a.H * (a.dB / fpk::BV);
-  hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a);
+  const int nwg = a.slots * a.H * (a.dB / fpk::BV) * (1 + (int)sizeof...(more));
+  hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a, more...);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     *err = hipGetErrorString(e);
@@ -106,7 +117,19 @@ struct DeviceRun {
   const char** err;
   template <int DA, int MODE, int NH>
   int go(int slot) const {
-    return launch(retention_pass_ws_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA), slot, a, stream, err);
+    return launch(retention_pass_ws_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA), slot, stream, err, a);
+  }
+};
+
+struct DevicePairRun {
+  const fpk::PassArgs& a;
+  const fpk::PassArgs& b;
+  hipStream_t stream;
+  const char** err;
+  template <int DA, int MODE, int NH>
+  int go(int slot) const {
+    return launch(retention_pass_pair_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA),
+                  fpk::PASS_KERNELS + slot, stream, err, a, fpk::tensors_of(b));
   }
 };
 
@@ -119,6 +142,19 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
     return 1;
   }
   return fpk::dispatch_pass(a, DeviceRun{a, static_cast<hipStream_t>(stream), err});
+}
+
+int fpk_launch_pass_pair(const fpk::PassArgs& first, const fpk::PassArgs& second, void* stream, const char** err) {
+  fpk::PassArgs a = first, b = second;
+  const int cus = fpk_compute_units();
+  const char* why = fpk::plan_pass(a, cus);
+  if (!why) why = fpk::plan_pass(b, cus);
+  if (!why && !fpk::same_walk(a, b)) why = "paired passes must walk the same shape the same way";
+  if (why) {
+    *err = why;
+    return 1;
+  }
+  return fpk::dispatch_pass(a, DevicePairRun{a, b, static_cast<hipStream_t>(stream), err});
 }
 
 int fpk_launch_scan(const fpk::ScanArgs& a, void* stream, const char** err) {

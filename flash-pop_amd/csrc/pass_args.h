@@ -51,6 +51,26 @@ struct PassArgs {
   float log2g[MAX_HEADS];
 };
 
+// The tensors of a pass without the rest of its arguments (what differs between two passes that
+// share a launch).
+struct PassTensors {
+  const uint16_t *X, *W, *Z;
+  uint16_t* Y;
+  const uint16_t* R0;
+  uint16_t *Rout, *Bout;
+  const uint16_t *Bin, *Xs, *Ws, *Zs;
+  uint16_t* Ys;
+  long long rs_a, rs_n;
+};
+#if defined(__HIPCC__)
+#define FPK_HOST_DEVICE __host__ __device__
+#else
+#define FPK_HOST_DEVICE
+#endif
+FPK_HOST_DEVICE inline PassTensors tensors_of(const PassArgs& a) {
+  return PassTensors{a.X, a.W, a.Z, a.Y, a.R0, a.Rout, a.Bout, a.Bin, a.Xs, a.Ws, a.Zs, a.Ys, a.rs_a, a.rs_n};
+}
+
 // Arguments of the segment scan that stitches a sequence cut into S segments back together.
 // U[b][s] is the state a segment contributes on its own (zero initial state); with g = gamma^Tseg
 //   init[b][0] = R0[b] (zeros if null),  init[b][s] = g init[b][s-1] + U[b][s-1],
@@ -123,6 +143,11 @@ constexpr int LAYER_THREADS = 256;
 // Launches the pass kernel on `stream` (a hipStream_t, or ignored by the CPU test harness).
 // Returns 0 on success; on failure returns nonzero and *err points at a static message.
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err);
+
+// Launches two passes that walk the same shape in the same direction in one grid, so that the
+// workgroups of a stream in both passes run side by side and share their reads of the tensors
+// the passes have in common.  The passes must not depend on each other.
+int fpk_launch_pass_pair(const fpk::PassArgs& a, const fpk::PassArgs& b, void* stream, const char** err);
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);

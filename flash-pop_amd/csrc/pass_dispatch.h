@@ -1,6 +1,8 @@
 // Validation of one pass launch and the choice of kernel instantiation, shared by the device
 // launcher and the CPU thread harness so that both take the same decisions.
 #pragma once
+#include <cstring>
+
 #include "pass_args.h"
 #include "retention_pass_ws.h"
 
@@ -40,6 +42,30 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
   if (a.slots < a.B && (!narrow || blocks || suffix))
     return "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
   return nullptr;
+}
+
+// Consecutive workgroup numbers go to the 8 XCDs in turn, and each XCD has an L2 of its own.  The
+// workgroups that read the same rows should meet in one L2: the column tiles of a stream and, in a
+// launch that holds two passes over the same tensors, the two passes of a stream.  Launch index
+// `block` of `passes * nwg` -> which pass (0 .. passes - 1) and which of its nwg workgroups.
+struct WorkgroupId {
+  int pass, wg;
+};
+FP_DEVICE WorkgroupId place_workgroup(int block, int nwg, int passes) {
+  if ((nwg & 7) != 0) return WorkgroupId{block % passes, block / passes};
+  const int xcd = block & 7, j = block >> 3;   // j-th workgroup that lands on this XCD
+  return WorkgroupId{j % passes, xcd * (nwg >> 3) + j / passes};
+}
+
+// Two passes can share a launch if they walk the same shape in the same way with the same
+// scalars (then they are the same kernel instantiation with the same grid, and differ in their
+// tensors only).
+inline bool same_walk(const PassArgs& a, const PassArgs& b) {
+  return a.B == b.B && a.T == b.T && a.H == b.H && a.dA == b.dA && a.dB == b.dB && a.nblk == b.nblk &&
+         a.block == b.block && a.reverse == b.reverse && a.Ls == b.Ls && a.state_only == b.state_only &&
+         a.slots == b.slots && (a.Bout != nullptr || a.Bin != nullptr) == (b.Bout != nullptr || b.Bin != nullptr) &&
+         a.s_intra == b.s_intra && a.s_read == b.s_read && a.s_update == b.s_update &&
+         std::memcmp(a.log2g, b.log2g, sizeof a.log2g) == 0;
 }
 
 // Calls run.template go<DA, MODE, NH>(slot) for the instantiation a planned `a` needs; `slot`

@@ -83,7 +83,10 @@ enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WA
 // accumulating across the two visits and convert, multiply by Z and store only after the second;
 // the state waves carry one set of accumulators per half and update the half being visited.
 template <int DA, int MODE, int NH = 1>
-FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
+// `nwg` workgroups run this pass and this one is number `wg` of them (the launch may hold the
+// workgroups of a second pass as well).  `io` are the tensors of this pass, by value: in a launch
+// of two passes they are chosen per workgroup, everything else in `p` is common to both.
+FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char* lds, int wg, int nwg) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
   static_assert(NH == 1 || (NH == 2 && (MODE == WALK_PLAIN || MODE == WALK_BLOCKS)), "two halves: plain and block walks only");
   constexpr bool STATE = MODE == WALK_STATE;
@@ -112,9 +115,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const int g = lane >> 5, c = lane & 31;
 
   const int ntile = p.dB / BV;
-  const int nwg = fprt::grid_size();
-  int wg = fprt::block_index();
-  if ((nwg & 7) == 0) wg = (wg & 7) * (nwg >> 3) + (wg >> 3);   // column tiles of a stream share an XCD
   const int tile = wg % ntile;
   const int h = (wg / ntile) % p.H;
   const int slot = (wg / ntile) / p.H;   // first batch entry of this workgroup
@@ -262,12 +262,12 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const float wread_fwd = p.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
 
     // ---- feeding X, Z and draining Y: coordinates of this thread, bytes from the chunk's first row
-    const char* const Xg = reinterpret_cast<const char*>(p.X);
-    const char* const Zg = reinterpret_cast<const char*>(p.Z);
-    char* const Yg = reinterpret_cast<char*>(p.Y);
-    const char* const Xsg = reinterpret_cast<const char*>(p.Xs);
-    const char* const Zsg = reinterpret_cast<const char*>(p.Zs);
-    char* const Ysg = reinterpret_cast<char*>(p.Ys);
+    const char* const Xg = reinterpret_cast<const char*>(io.X);
+    const char* const Zg = reinterpret_cast<const char*>(io.Z);
+    char* const Yg = reinterpret_cast<char*>(io.Y);
+    const char* const Xsg = reinterpret_cast<const char*>(io.Xs);
+    const char* const Zsg = reinterpret_cast<const char*>(io.Zs);
+    char* const Ysg = reinterpret_cast<char*>(io.Ys);
     uint32_t xg_off[NXP];
     int xs_off[NXP];
 #pragma unroll
@@ -528,8 +528,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   const bool ws_writer = NAB == 4 || (sub & 1) == 0; // one wave per row block fills the row-major W tile
   uint16_t* const wt = WT + sub * 32 * T_LD;
 
-  const char* const Wg = reinterpret_cast<const char*>(p.W);
-  const char* const Wsg = reinterpret_cast<const char*>(p.Ws);
+  const char* const Wg = reinterpret_cast<const char*>(io.W);
+  const char* const Wsg = reinterpret_cast<const char*>(io.Ws);
   const size_t mat = (size_t)p.dA * p.dB;
 
   // per-thread coordinates, bytes relative to the chunk's first row; they never change
@@ -570,7 +570,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   // the staging area the tile is kept in the order of the global matrix: for R = S that is
   // [a][n] (one accumulator element per 2-byte access), for R = S^T it is [n][a], which is also
   // the natural order of the staging buffer (four accumulator elements per 8-byte access).
-  const bool tposed = p.rs_a == 1;
+  const bool tposed = io.rs_a == 1;
   constexpr int NP = 2 * NNW;                    // 16-byte pieces per lane
   constexpr int NCOL = 32 * NNW;                 // tile columns
   struct TileRegs {
@@ -589,16 +589,16 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     const int q = lane + 64 * u;
     if (!tposed) {
       const int a_l = q / (4 * NNW), piece = q % (4 * NNW);
-      tile_goff[u] = 2u * (uint32_t)((32 * ablk + a_l) * (int)p.rs_a + tile * BV + 32 * nb0 + 8 * piece);
+      tile_goff[u] = 2u * (uint32_t)((32 * ablk + a_l) * (int)io.rs_a + tile * BV + 32 * nb0 + 8 * piece);
       tile_soff[u] = stage_elem(a_l * NCOL + 8 * piece);
     } else {
       const int n_l = q / 4, piece = q % 4;
-      tile_goff[u] = 2u * (uint32_t)((tile * BV + 32 * nb0 + n_l) * (int)p.rs_n + 32 * ablk + 8 * piece);
+      tile_goff[u] = 2u * (uint32_t)((tile * BV + 32 * nb0 + n_l) * (int)io.rs_n + 32 * ablk + 8 * piece);
       tile_soff[u] = stage_elem(n_l * 32 + 8 * piece);
     }
   }
   // byte offset of half hf of the rows of R inside a state matrix
-  const uint32_t half_stride = 2u * DA * (uint32_t)(tposed ? 1 : p.rs_a);
+  const uint32_t half_stride = 2u * DA * (uint32_t)(tposed ? 1 : io.rs_a);
   // issue the global loads of a tile; `src` null or !live -> zeros without memory traffic
   auto tile_load = [&](TileRegs& tr, const uint16_t* src, bool live, int hf) {
     const fprt::BufView view = fprt::make_buf(src, (src && live) ? (uint32_t)(mat * 2) : 0u);
@@ -721,10 +721,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
   for (int hf = 0; hf < NH; ++hf) {
     // initial R, plus the gradient of the last block state if the first chunk of a reverse pass ends a block
     TileRegs t_init, t_inj;
-    tile_load(t_init, p.R0 ? state_matrix(p.R0, cur.b) : nullptr, true, hf);
-    const bool inj = BLOCKS && p.Bin && ends_block(cur.t0 + cur.L);
-    tile_load(t_inj, inj ? block_matrix(p.Bin, cur.b, cur.t0 + cur.L) : nullptr, inj, hf);
-    if (p.R0) tile_accumulate(t_init, 0, false, racc[hf]);
+    tile_load(t_init, io.R0 ? state_matrix(io.R0, cur.b) : nullptr, true, hf);
+    const bool inj = BLOCKS && io.Bin && ends_block(cur.t0 + cur.L);
+    tile_load(t_inj, inj ? block_matrix(io.Bin, cur.b, cur.t0 + cur.L) : nullptr, inj, hf);
+    if (io.R0) tile_accumulate(t_init, 0, false, racc[hf]);
     if (inj) tile_accumulate(t_inj, 0, true, racc[hf]);
   }
   write_rt(0, racc[0]);
@@ -746,16 +746,16 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     fprt::prof_stamp(it, 0);
     const Chunk nn = chunk_after(nxt);
     // gradient of the block state that the next chunk ends (reverse pass); an empty view otherwise
-    const bool inj = BLOCKS && closes && p.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
+    const bool inj = BLOCKS && closes && io.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
     TileRegs t_inj[NH];
     if (BLOCKS && closes) {
 #pragma unroll
-      for (int hf = 0; hf < NH; ++hf) tile_load(t_inj[hf], inj ? block_matrix(p.Bin, nxt.b, nxt.t0 + nxt.L) : nullptr, inj, hf);
+      for (int hf = 0; hf < NH; ++hf) tile_load(t_inj[hf], inj ? block_matrix(io.Bin, nxt.b, nxt.t0 + nxt.L) : nullptr, inj, hf);
     }
     // initial state of the next sequence, if the next chunk starts one
     const bool fresh = MULTI && nxt.ok && nxt.first;
     TileRegs t_init;
-    if (MULTI) tile_load(t_init, (fresh && p.R0) ? state_matrix(p.R0, nxt.b) : nullptr, fresh, 0);
+    if (MULTI) tile_load(t_init, (fresh && io.R0) ? state_matrix(io.R0, nxt.b) : nullptr, fresh, 0);
 
     if (dbg & 4) {
       if (!STATE && closes) fprt::block_sync();
@@ -842,15 +842,15 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, char* lds) {
     if (closes) {
 #pragma unroll
       for (int hf = 0; hf < NH; ++hf) {
-        if (BLOCKS && p.Bout && ends_block(t1))
-          tile_store(const_cast<uint16_t*>(block_matrix(p.Bout, cur.b, t1)), s ^ 1, racc[hf], hf);
-        if (cur.last && p.Rout) tile_store(const_cast<uint16_t*>(state_matrix(p.Rout, cur.b)), s ^ 1, racc[hf], hf);
+        if (BLOCKS && io.Bout && ends_block(t1))
+          tile_store(const_cast<uint16_t*>(block_matrix(io.Bout, cur.b, t1)), s ^ 1, racc[hf], hf);
+        if (cur.last && io.Rout) tile_store(const_cast<uint16_t*>(state_matrix(io.Rout, cur.b)), s ^ 1, racc[hf], hf);
       }
     }
     fprt::prof_stamp(it, 3);
     if (nxt.ok) {
       if (MULTI && fresh) {
-        if (p.R0) {
+        if (io.R0) {
           tile_accumulate(t_init, s ^ 1, false, racc[0]);
         } else {
 #pragma unroll

@@ -53,7 +53,22 @@ struct HarnessRun {
   template <int DA, int MODE, int NH>
   int go(int /*slot*/) const {
     const int nwg = a.slots * a.H * (a.dB / fpk::BV);
-    return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(DA), [&](char* l) { fpk::retention_pass_ws<DA, MODE, NH>(a, l); });
+    return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(DA), [&](char* l) {
+      fpk::retention_pass_ws<DA, MODE, NH>(a, fpk::tensors_of(a), l, fpk::place_workgroup(fprt::block_index(), nwg, 1).wg, nwg);
+    });
+  }
+};
+
+struct HarnessPairRun {
+  const fpk::PassArgs& a;
+  const fpk::PassArgs& b;
+  template <int DA, int MODE, int NH>
+  int go(int /*slot*/) const {
+    const int nwg = a.slots * a.H * (a.dB / fpk::BV);
+    return run_grid(fpk::NTHREADS_WS, 2 * nwg, fpk::lds_bytes_ws(DA), [&](char* l) {
+      const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, 2);
+      fpk::retention_pass_ws<DA, MODE, NH>(a, fpk::tensors_of(id.pass ? b : a), l, id.wg, nwg);
+    });
   }
 };
 
@@ -66,6 +81,18 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
     return 1;
   }
   return fpk::dispatch_pass(a, HarnessRun{a});
+}
+
+int fpk_launch_pass_pair(const fpk::PassArgs& first, const fpk::PassArgs& second, void* /*stream*/, const char** err) {
+  fpk::PassArgs a = first, b = second;
+  const char* why = fpk::plan_pass(a, fpk_compute_units());
+  if (!why) why = fpk::plan_pass(b, fpk_compute_units());
+  if (!why && !fpk::same_walk(a, b)) why = "paired passes must walk the same shape the same way";
+  if (why) {
+    *err = why;
+    return 1;
+  }
+  return fpk::dispatch_pass(a, HarnessPairRun{a, b});
 }
 
 // Pretends the chip has 8 compute units, so that small test shapes take the paths that large
