@@ -104,7 +104,7 @@ def gpu_leg(args):
         "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": {
             "bound": "hbm",
-            "kernel": "retention_pass_ws_kernel<128, 0, 1> (forward, dq) and retention_pass_pair_kernel<128, 0, 1> "
+            "kernel": "retention_pass_ws_kernel<128, 0, 1> (forward, dq) and retention_pass_multi_kernel<128, 0, 1> "
                       "(dk and dv passes in one launch)",
             "achieved": round(achieved_gbs, 1),
             "peak": HBM_PEAK_GBS,

@@ -11,8 +11,8 @@
 //
 // The column dimension dB is split over workgroups, the contraction dimension dA never is,
 // so no pass needs a cross-workgroup reduction.  The dq pass re-runs the state recurrence
-// instead of reading stored chunk states; the dk and dv passes each carry dS and, when dk == dv,
-// share one launch so that the q and dO rows both of them read come from HBM once.
+// instead of reading stored chunk states; the dk and dv passes each carry dS.  The three gradient
+// passes are independent of each other and share launches where they fit (run_gradients).
 //
 // The POP entry points add block states to these passes (written by fwd, their gradients read
 // by dk and dv); the fused POP entry points add the suffix tensors in the same four roles; the
@@ -88,17 +88,58 @@ int run(const fpk::PassArgs& a, void* stream, const char* what) {
   return FP_OK;
 }
 
-// The dk and dv passes read the same q and dO rows walking in the same direction.  When dk == dv
-// they are the same kernel with the same grid, and one launch runs the workgroups of a stream in
-// both passes side by side: q and dO then come from HBM once instead of twice.
-int run_dk_dv(const fpk::PassArgs& pass_dk, const fpk::PassArgs& pass_dv, void* stream, const char* what) {
-  if (pass_dk.dA != pass_dv.dA) {
-    if (int rc = run(pass_dk, stream, what)) return rc;
-    return run(pass_dv, stream, what);
-  }
+// Independent passes over the same shape may share a launch (fpk_launch_passes).
+bool same_launch(const fpk::PassArgs& x, const fpk::PassArgs& y) {
+  return x.dA == y.dA && x.dB == y.dB && x.block == y.block && x.nblk == y.nblk && x.Ls == y.Ls &&
+         (x.Bin != nullptr || x.Bout != nullptr) == (y.Bin != nullptr || y.Bout != nullptr);
+}
+
+int run_together(const fpk::PassArgs* const* passes, int n, void* stream, const char* what) {
   const char* msg = "";
-  if (fpk_launch_pass_pair(pass_dk, pass_dv, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s passes: %s", what, msg);
+  if (fpk_launch_passes(passes, n, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s passes: %s", what, msg);
   return FP_OK;
+}
+
+// The three gradient passes do not depend on each other.  How they are grouped into launches:
+//  - dk and dv read the same q and dO rows walking backward; with dk == dv they are the same
+//    kernel with the same grid, and in one launch the workgroups of a stream in both passes run
+//    side by side, so those rows come from HBM once;
+//  - dq has the shape of the dk pass.  Where one pass alone leaves compute units idle it joins
+//    that launch (it walks the other way, so nothing is shared but the chip);
+//  - what does not fit together (different dk and dv; block states in dk and dv but not in dq)
+//    is launched on its own.
+int run_gradients(const fpk::PassArgs& dq, const fpk::PassArgs& dk, const fpk::PassArgs& dv, void* stream,
+                  const char* what) {
+  const long long alone = (long long)dk.B * dk.H * (dk.dB / fpk::BV);   // workgroups of one pass
+  const bool fills = alone >= fpk_compute_units();
+  const bool dq_dk = same_launch(dq, dk), dk_dv = same_launch(dk, dv);
+  if (dq_dk && dk_dv && !fills) {
+    const fpk::PassArgs* all[] = {&dk, &dv, &dq};
+    return run_together(all, 3, stream, what);
+  }
+  if (dk_dv) {
+    if (int rc = run(dq, stream, what)) return rc;
+    const fpk::PassArgs* both[] = {&dk, &dv};
+    return run_together(both, 2, stream, what);
+  }
+  if (dq_dk && !fills) {
+    const fpk::PassArgs* both[] = {&dq, &dk};
+    if (int rc = run_together(both, 2, stream, what)) return rc;
+    return run(dv, stream, what);
+  }
+  if (int rc = run(dq, stream, what)) return rc;
+  if (int rc = run(dk, stream, what)) return rc;
+  return run(dv, stream, what);
+}
+
+// dk and dv alone (the split-sequence backward runs its dq earlier)
+int run_dk_dv(const fpk::PassArgs& dk, const fpk::PassArgs& dv, void* stream, const char* what) {
+  if (same_launch(dk, dv)) {
+    const fpk::PassArgs* both[] = {&dk, &dv};
+    return run_together(both, 2, stream, what);
+  }
+  if (int rc = run(dk, stream, what)) return rc;
+  return run(dv, stream, what);
 }
 
 // R = S, dk x dv, rows contiguous in dv
@@ -136,16 +177,14 @@ int backward(const Shape& s, const void* q, const void* k, const void* v, const 
              void* d_s0, void* stream) {
   const float sc = 1.0f / std::sqrt((float)s.dk);
   const int nblk = block > 0 ? s.T / block : 0;
-  fpk::PassArgs a;
-  int rc;
+  fpk::PassArgs g, a;
 
-  fill_common(a, s, decays);   // dq
-  a.X = in(d_o); a.W = in(v); a.Z = in(k); a.Y = out(dq);
-  a.R0 = in(s0);
-  transposed_state(a, s);
-  a.reverse = 0;
-  a.s_intra = sc; a.s_read = 1.f; a.s_update = sc;
-  if ((rc = run(a, stream, "dq")) != FP_OK) return rc;
+  fill_common(g, s, decays);   // dq
+  g.X = in(d_o); g.W = in(v); g.Z = in(k); g.Y = out(dq);
+  g.R0 = in(s0);
+  transposed_state(g, s);
+  g.reverse = 0;
+  g.s_intra = sc; g.s_read = 1.f; g.s_update = sc;
 
   fill_common(a, s, decays);   // dk
   a.X = in(v); a.W = in(d_o); a.Z = in(q); a.Y = out(dk_);
@@ -163,7 +202,7 @@ int backward(const Shape& s, const void* q, const void* k, const void* v, const 
   b.block = d_blocks ? block : 0; b.nblk = nblk;
   b.reverse = 1;
   b.s_intra = sc; b.s_read = sc; b.s_update = 1.f;
-  return run_dk_dv(a, b, stream, "dk / dv");
+  return run_gradients(g, a, b, stream, "gradient");
 }
 
 // ---- long sequences, few streams: cut every sequence into segments ---------------------------
@@ -347,17 +386,15 @@ int fused_backward(const Shape& s, const void* q, const void* k, const void* v, 
                    const double* decays, const void* d_o, const void* d_o_sfx, const void* d_s_out, void* dq, void* dk_,
                    void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx, void* d_s0, int block, void* stream) {
   const float sc = 1.0f / std::sqrt((float)s.dk);
-  fpk::PassArgs a;
-  int rc;
+  fpk::PassArgs g, a;
 
-  fill_common(a, s, decays);   // dq
-  a.X = in(d_o); a.W = in(v); a.Z = in(k); a.Y = out(dq);
-  a.R0 = in(s0);
-  transposed_state(a, s);
-  suffix_walk(a, s, block, x.len, d_o_sfx, x.v, x.k, dq_sfx);
-  a.reverse = 0;
-  a.s_intra = sc; a.s_read = 1.f; a.s_update = sc;
-  if ((rc = run(a, stream, "fused dq")) != FP_OK) return rc;
+  fill_common(g, s, decays);   // dq
+  g.X = in(d_o); g.W = in(v); g.Z = in(k); g.Y = out(dq);
+  g.R0 = in(s0);
+  transposed_state(g, s);
+  suffix_walk(g, s, block, x.len, d_o_sfx, x.v, x.k, dq_sfx);
+  g.reverse = 0;
+  g.s_intra = sc; g.s_read = 1.f; g.s_update = sc;
 
   fill_common(a, s, decays);   // dk
   a.X = in(v); a.W = in(d_o); a.Z = in(q); a.Y = out(dk_);
@@ -375,7 +412,7 @@ int fused_backward(const Shape& s, const void* q, const void* k, const void* v, 
   suffix_walk(b, s, block, x.len, x.k, x.q, d_o_sfx, dv_sfx);
   b.reverse = 1;
   b.s_intra = sc; b.s_read = sc; b.s_update = 1.f;
-  return run_dk_dv(a, b, stream, "fused dk / dv");
+  return run_gradients(g, a, b, stream, "fused gradient");
 }
 
 }  // namespace

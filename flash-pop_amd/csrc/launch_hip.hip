@@ -17,14 +17,17 @@ __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_ws_kernel(con
   fpk::retention_pass_ws<DA, MODE, NH>(args, fpk::tensors_of(args), lds, fpk::place_workgroup(fprt::block_index(), nwg, 1).wg, nwg);
 }
 
-// Two independent passes of the same shape in one grid (see fpk_launch_pass_pair).
+// Up to three independent passes over the same shape in one grid (see fpk_launch_passes).
 template <int DA, int MODE, int NH = 1>
-__global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_pair_kernel(const fpk::PassArgs first,
-                                                                               const fpk::PassTensors second) {
+__global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_multi_kernel(const fpk::PassArgs first,
+                                                                                const fpk::PassTensors second,
+                                                                                const fpk::PassTensors third,
+                                                                                const int passes) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int nwg = fprt::grid_size() / 2;
-  const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, 2);
-  fpk::retention_pass_ws<DA, MODE, NH>(first, id.pass ? second : fpk::tensors_of(first), lds, id.wg, nwg);
+  const int nwg = fprt::grid_size() / passes;
+  const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, passes);
+  const fpk::PassTensors io = id.pass == 0 ? fpk::tensors_of(first) : id.pass == 1 ? second : third;
+  fpk::retention_pass_ws<DA, MODE, NH>(first, io, lds, id.wg, nwg);
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -56,9 +59,9 @@ constexpr int kMaxDevices = 64;
 static_assert(2 * fpk::PASS_KERNELS <= 32, "one bit per kernel instantiation, single and paired");
 std::atomic<uint32_t> g_armed[kMaxDevices];
 
-template <typename Kernel, typename... Second>
-int launch(Kernel kernel, int threads, int lds, int slot, hipStream_t stream, const char** err, const fpk::PassArgs& a,
-           const Second&... more) {
+template <typename Kernel, typename... More>
+int launch(Kernel kernel, int threads, int lds, int slot, int passes, hipStream_t stream, const char** err,
+           const fpk::PassArgs& a, const More&... more) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     *err = "hipGetDevice failed";
@@ -74,7 +77,7 @@ int launch(Kernel kernel, int threads, int lds, int slot, hipStream_t stream, co
     }
     if (tracked) g_armed[dev].fetch_or(1u << slot, std::memory_order_release);
   }
-  const int nwg = a.slots * a.H * (a.dB / fpk::BV) * (1 + (int)sizeof...(more));
+  const int nwg = a.slots * a.H * (a.dB / fpk::BV) * passes;
   hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a, more...);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -117,19 +120,20 @@ struct DeviceRun {
   const char** err;
   template <int DA, int MODE, int NH>
   int go(int slot) const {
-    return launch(retention_pass_ws_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA), slot, stream, err, a);
+    return launch(retention_pass_ws_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA), slot, 1, stream, err, a);
   }
 };
 
-struct DevicePairRun {
-  const fpk::PassArgs& a;
-  const fpk::PassArgs& b;
+struct DeviceMultiRun {
+  const fpk::PassArgs* planned;
+  int n;
   hipStream_t stream;
   const char** err;
   template <int DA, int MODE, int NH>
   int go(int slot) const {
-    return launch(retention_pass_pair_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA),
-                  fpk::PASS_KERNELS + slot, stream, err, a, fpk::tensors_of(b));
+    return launch(retention_pass_multi_kernel<DA, MODE, NH>, fpk::NTHREADS_WS, fpk::lds_bytes_ws(DA),
+                  fpk::PASS_KERNELS + slot, n, stream, err, planned[0], fpk::tensors_of(planned[1]),
+                  fpk::tensors_of(planned[n - 1]), n);
   }
 };
 
@@ -144,17 +148,14 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err) {
   return fpk::dispatch_pass(a, DeviceRun{a, static_cast<hipStream_t>(stream), err});
 }
 
-int fpk_launch_pass_pair(const fpk::PassArgs& first, const fpk::PassArgs& second, void* stream, const char** err) {
-  fpk::PassArgs a = first, b = second;
-  const int cus = fpk_compute_units();
-  const char* why = fpk::plan_pass(a, cus);
-  if (!why) why = fpk::plan_pass(b, cus);
-  if (!why && !fpk::same_walk(a, b)) why = "paired passes must walk the same shape the same way";
-  if (why) {
+int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, const char** err) {
+  if (n == 1) return fpk_launch_pass(*passes[0], stream, err);
+  fpk::PassArgs planned[fpk::MAX_PASSES_PER_LAUNCH];
+  if (const char* why = fpk::plan_passes(planned, passes, n, fpk_compute_units())) {
     *err = why;
     return 1;
   }
-  return fpk::dispatch_pass(a, DevicePairRun{a, b, static_cast<hipStream_t>(stream), err});
+  return fpk::dispatch_pass(planned[0], DeviceMultiRun{planned, n, static_cast<hipStream_t>(stream), err});
 }
 
 int fpk_launch_scan(const fpk::ScanArgs& a, void* stream, const char** err) {

@@ -51,8 +51,8 @@ struct PassArgs {
   float log2g[MAX_HEADS];
 };
 
-// The tensors of a pass without the rest of its arguments (what differs between two passes that
-// share a launch).
+// What can differ between passes that share a launch: the tensors, the walking direction and the
+// three scales.  Everything else in PassArgs (shape, walk, decays) is common to them.
 struct PassTensors {
   const uint16_t *X, *W, *Z;
   uint16_t* Y;
@@ -61,6 +61,8 @@ struct PassTensors {
   const uint16_t *Bin, *Xs, *Ws, *Zs;
   uint16_t* Ys;
   long long rs_a, rs_n;
+  int reverse;
+  float s_intra, s_read, s_update;
 };
 #if defined(__HIPCC__)
 #define FPK_HOST_DEVICE __host__ __device__
@@ -68,8 +70,11 @@ struct PassTensors {
 #define FPK_HOST_DEVICE
 #endif
 FPK_HOST_DEVICE inline PassTensors tensors_of(const PassArgs& a) {
-  return PassTensors{a.X, a.W, a.Z, a.Y, a.R0, a.Rout, a.Bout, a.Bin, a.Xs, a.Ws, a.Zs, a.Ys, a.rs_a, a.rs_n};
+  return PassTensors{a.X,  a.W,  a.Z,  a.Y,    a.R0,   a.Rout,    a.Bout,    a.Bin,    a.Xs,
+                     a.Ws, a.Zs, a.Ys, a.rs_a, a.rs_n, a.reverse, a.s_intra, a.s_read, a.s_update};
 }
+
+constexpr int MAX_PASSES_PER_LAUNCH = 3;
 
 // Arguments of the segment scan that stitches a sequence cut into S segments back together.
 // U[b][s] is the state a segment contributes on its own (zero initial state); with g = gamma^Tseg
@@ -144,10 +149,12 @@ constexpr int LAYER_THREADS = 256;
 // Returns 0 on success; on failure returns nonzero and *err points at a static message.
 int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err);
 
-// Launches two passes that walk the same shape in the same direction in one grid, so that the
-// workgroups of a stream in both passes run side by side and share their reads of the tensors
-// the passes have in common.  The passes must not depend on each other.
-int fpk_launch_pass_pair(const fpk::PassArgs& a, const fpk::PassArgs& b, void* stream, const char** err);
+// Launches n <= MAX_PASSES_PER_LAUNCH independent passes over the same shape in one grid (they
+// must be the same walk of the same shape; tensors, direction and scales may differ).  A pass that
+// would leave part of the chip idle on its own runs beside the others, and passes that read the
+// same rows in the same direction have the workgroups of a stream run side by side, so that those
+// rows come from HBM once.
+int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, const char** err);
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);

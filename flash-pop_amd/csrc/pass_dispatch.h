@@ -46,7 +46,7 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
 
 // Consecutive workgroup numbers go to the 8 XCDs in turn, and each XCD has an L2 of its own.  The
 // workgroups that read the same rows should meet in one L2: the column tiles of a stream and, in a
-// launch that holds two passes over the same tensors, the two passes of a stream.  Launch index
+// launch that holds several passes over the same tensors, the passes of a stream.  Launch index
 // `block` of `passes * nwg` -> which pass (0 .. passes - 1) and which of its nwg workgroups.
 struct WorkgroupId {
   int pass, wg;
@@ -57,15 +57,24 @@ FP_DEVICE WorkgroupId place_workgroup(int block, int nwg, int passes) {
   return WorkgroupId{j % passes, xcd * (nwg >> 3) + j / passes};
 }
 
-// Two passes can share a launch if they walk the same shape in the same way with the same
-// scalars (then they are the same kernel instantiation with the same grid, and differ in their
-// tensors only).
+// Passes can share a launch if they walk the same shape in the same way (then they are the same
+// kernel instantiation with the same grid); their tensors, direction and scales may differ.
 inline bool same_walk(const PassArgs& a, const PassArgs& b) {
   return a.B == b.B && a.T == b.T && a.H == b.H && a.dA == b.dA && a.dB == b.dB && a.nblk == b.nblk &&
-         a.block == b.block && a.reverse == b.reverse && a.Ls == b.Ls && a.state_only == b.state_only &&
-         a.slots == b.slots && (a.Bout != nullptr || a.Bin != nullptr) == (b.Bout != nullptr || b.Bin != nullptr) &&
-         a.s_intra == b.s_intra && a.s_read == b.s_read && a.s_update == b.s_update &&
+         a.block == b.block && a.Ls == b.Ls && a.state_only == b.state_only && a.slots == b.slots &&
+         (a.Bout != nullptr || a.Bin != nullptr) == (b.Bout != nullptr || b.Bin != nullptr) &&
          std::memcmp(a.log2g, b.log2g, sizeof a.log2g) == 0;
+}
+
+// Plans every pass of a launch and checks that they fit together.  Returns nullptr or a message.
+inline const char* plan_passes(PassArgs* planned, const PassArgs* const* passes, int n, int compute_units) {
+  if (n < 1 || n > MAX_PASSES_PER_LAUNCH) return "a launch holds one to three passes";
+  for (int i = 0; i < n; ++i) {
+    planned[i] = *passes[i];
+    if (const char* why = plan_pass(planned[i], compute_units)) return why;
+    if (i > 0 && !same_walk(planned[0], planned[i])) return "passes that share a launch must walk the same shape the same way";
+  }
+  return nullptr;
 }
 
 // Calls run.template go<DA, MODE, NH>(slot) for the instantiation a planned `a` needs; `slot`

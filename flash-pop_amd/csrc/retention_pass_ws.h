@@ -84,8 +84,9 @@ enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WA
 // the state waves carry one set of accumulators per half and update the half being visited.
 template <int DA, int MODE, int NH = 1>
 // `nwg` workgroups run this pass and this one is number `wg` of them (the launch may hold the
-// workgroups of a second pass as well).  `io` are the tensors of this pass, by value: in a launch
-// of two passes they are chosen per workgroup, everything else in `p` is common to both.
+// workgroups of other passes as well).  `io` are the tensors, walking direction and scales of
+// this pass, by value: in a launch of several passes they are chosen per workgroup, everything
+// else in `p` is common to all of them.
 FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char* lds, int wg, int nwg) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
   static_assert(NH == 1 || (NH == 2 && (MODE == WALK_PLAIN || MODE == WALK_BLOCKS)), "two halves: plain and block walks only");
@@ -122,7 +123,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   const int dbg = fprt::dbg_flags();   // always 0 outside profiling builds
   const int T = p.T;
   const int bs = (BLOCKS || SFX) ? p.block : 0;   // only these walks cut chunks at block boundaries
-  const bool rev = p.reverse != 0;
+  const bool rev = io.reverse != 0;
   const float lg = p.log2g[h];
 
   // chunk [t0, t0 + L) that follows position `pos` in walking order; never straddles a block boundary
@@ -241,7 +242,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     for (int r = 0; r < 16; ++r) {
       const int jl = acc_row(r, g);
       const int d = rev ? (jl - c) : (c - jl);          // distance inside the diagonal tile
-      mw[r] = p.s_intra * fprt::exp2_approx((float)(makes_diag ? (d >= 0 ? d : 0) : 32 + d) * lg);
+      mw[r] = io.s_intra * fprt::exp2_approx((float)(makes_diag ? (d >= 0 ? d : 0) : 32 + d) * lg);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -259,7 +260,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     const int zm_off = (32 * nb + c) * T_LD + 4 * g + 32 * (makes_diag ? ib : 1 - ib);
     const int zh_off = (32 * nb + c) * T_LD + 4 * g + 32 * (makes_diag ? 1 - ib : ib);
     const int y_off = i_row * YB_LD + 32 * nb + 4 * g;
-    const float wread_fwd = p.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
+    const float wread_fwd = io.s_read * fprt::exp2_approx((float)(i_row + 1) * lg);
 
     // ---- feeding X, Z and draining Y: coordinates of this thread, bytes from the chunk's first row
     const char* const Xg = reinterpret_cast<const char*>(io.X);
@@ -370,7 +371,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       if (rev) {
         int e = L - 1 - i_row;
         if (e < 0) e = 0;
-        wread = p.s_read * fprt::exp2_approx((float)e * lg);
+        wread = io.s_read * fprt::exp2_approx((float)e * lg);
         if (SFX && ck.sfx) wread = 0.f;   // nothing downstream of a suffix reaches back into it
       }
 
@@ -695,7 +696,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
         const int j = 4 * w_tg + r;
         int e = rev ? (j + 1) : (ck.L - 1 - j);
         if (e < 0) e = 0;
-        wkey[r] = p.s_update * fprt::exp2_approx((float)e * lg);
+        wkey[r] = io.s_update * fprt::exp2_approx((float)e * lg);
       }
     }
 #pragma unroll

@@ -59,15 +59,16 @@ struct HarnessRun {
   }
 };
 
-struct HarnessPairRun {
-  const fpk::PassArgs& a;
-  const fpk::PassArgs& b;
+struct HarnessMultiRun {
+  const fpk::PassArgs* planned;
+  int n;
   template <int DA, int MODE, int NH>
   int go(int /*slot*/) const {
+    const fpk::PassArgs& a = planned[0];
     const int nwg = a.slots * a.H * (a.dB / fpk::BV);
-    return run_grid(fpk::NTHREADS_WS, 2 * nwg, fpk::lds_bytes_ws(DA), [&](char* l) {
-      const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, 2);
-      fpk::retention_pass_ws<DA, MODE, NH>(a, fpk::tensors_of(id.pass ? b : a), l, id.wg, nwg);
+    return run_grid(fpk::NTHREADS_WS, n * nwg, fpk::lds_bytes_ws(DA), [&](char* l) {
+      const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, n);
+      fpk::retention_pass_ws<DA, MODE, NH>(a, fpk::tensors_of(planned[id.pass]), l, id.wg, nwg);
     });
   }
 };
@@ -83,16 +84,14 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
   return fpk::dispatch_pass(a, HarnessRun{a});
 }
 
-int fpk_launch_pass_pair(const fpk::PassArgs& first, const fpk::PassArgs& second, void* /*stream*/, const char** err) {
-  fpk::PassArgs a = first, b = second;
-  const char* why = fpk::plan_pass(a, fpk_compute_units());
-  if (!why) why = fpk::plan_pass(b, fpk_compute_units());
-  if (!why && !fpk::same_walk(a, b)) why = "paired passes must walk the same shape the same way";
-  if (why) {
+int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, const char** err) {
+  if (n == 1) return fpk_launch_pass(*passes[0], stream, err);
+  fpk::PassArgs planned[fpk::MAX_PASSES_PER_LAUNCH];
+  if (const char* why = fpk::plan_passes(planned, passes, n, fpk_compute_units())) {
     *err = why;
     return 1;
   }
-  return fpk::dispatch_pass(a, HarnessPairRun{a, b});
+  return fpk::dispatch_pass(planned[0], HarnessMultiRun{planned, n});
 }
 
 // Pretends the chip has 8 compute units, so that small test shapes take the paths that large
