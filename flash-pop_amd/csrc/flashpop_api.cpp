@@ -353,8 +353,6 @@ int check_fused(const Shape& s, int block, int sfx_len) {
     return fail(FP_ERR_BAD_SHAPE, "the fused POP op needs T to be a multiple of block_size (got T=%d, block_size=%d)", s.T, block);
   if (sfx_len < 1 || sfx_len > fpk::CH)
     return fail(FP_ERR_BAD_SHAPE, "suffix length must be in 1..%d (got %d)", fpk::CH, sfx_len);
-  if (s.dk > 128 || s.dv > 128)
-    return fail(FP_ERR_UNSUPPORTED_DIM, "the fused POP op supports dk and dv of 64 or 128 (got dk=%d, dv=%d)", s.dk, s.dv);
   if ((long long)s.B * (s.T / block + 1) * sfx_len >= (1LL << 32))
     return fail(FP_ERR_BAD_SHAPE, "too many suffix rows: B * (T / block_size + 1) * sfx_len must stay below 2^32");
   return FP_OK;

@@ -9,7 +9,7 @@
 namespace fpk {
 
 // Number of kernel instantiations `dispatch_pass` can pick from (its `slot` argument is below this).
-constexpr int PASS_KERNELS = 12;
+constexpr int PASS_KERNELS = 13;
 
 // Checks what the walks assume about `a` and chooses a.slots (workgroups per (head, column tile))
 // for a device with `compute_units` units.  Returns nullptr, or a message for the caller.
@@ -21,8 +21,8 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
   if (a.dB < BV || a.dB % BV != 0) return "dB must be a multiple of 64";
   if (suffix) {
     // the C-ABI layer reports these to the caller in its own words
-    if (!narrow || blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys)
-      return "suffix walk: needs dA of 64 or 128, T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
+    if (blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys)
+      return "suffix walk: needs T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
     a.slots = a.B;
   }
   // One workgroup per (batch entry, head, column tile) while that fits the chip once; beyond that
@@ -98,6 +98,7 @@ int dispatch_pass(const PassArgs& a, Run&& run) {
     return run.template go<128, WALK_PLAIN, 1>(9);
   }
   // dA = 256: two visits per chunk, 128 of the 256 contraction columns each
+  if (suffix) return run.template go<128, WALK_SUFFIX, 2>(12);
   if (blocks) return run.template go<128, WALK_BLOCKS, 2>(10);
   return run.template go<128, WALK_PLAIN, 2>(11);
 }

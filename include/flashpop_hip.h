@@ -98,7 +98,7 @@ int fp_pop_retention_bwd(const void* q, const void* k, const void* v, const void
  *                 index fastest, N = T / block_size, as the reference batches its suffixes
  *   s_out         out: state after the last block, the reference's `last_state` (pop_retnet.py:169);
  *                 may be NULL
- * Needs T % block_size == 0 (as the reference's layer does), 1 <= sfx_len <= 64 and dk, dv in {64, 128}. */
+ * Needs T % block_size == 0 (as the reference's layer does) and 1 <= sfx_len <= 64. */
 int fp_pop_fused_fwd(const void* q, const void* k, const void* v, const void* s0, const void* q_sfx, const void* k_sfx,
                      const void* v_sfx, const double* head_decays, void* o, void* o_sfx, void* s_out, int B, int T,
                      int H, int dk, int dv, int block_size, int sfx_len, void* stream);

@@ -123,6 +123,7 @@ int main() {
   rc |= pop(1, 96, 1, 256, 64, 32);           // block states with two visits per chunk
   rc |= fused(2, 2, 80, 5, 1, 64, 128);
   rc |= fused(1, 3, 24, 64, 1, 128, 64);
+  rc |= fused(1, 2, 40, 9, 1, 64, 256);       // suffixes with two visits per chunk
   rc |= decode(2, 3, 64, 128);
   rc |= decode(1, 1, 256, 256);
   rc |= rotary(3, 11, 2, 64, true);           // last workgroup partly idle

@@ -51,13 +51,13 @@ def test_argument_checks_return_codes(lib):
     bad0 = (ctypes.c_double * 2)(0.0, 0.5)
     assert lib.fp_retention_fwd(p, p, p, null, bad0, p, null, *ok_dims, None) == -4
     assert lib.fp_retention_bwd(p, p, p, null, dec, null, null, p, p, p, null, *ok_dims, None) == -1
-    # fused POP op: T a multiple of the block, suffix length 1..64, dims up to 128, no NULL tensors
+    # fused POP op: T a multiple of the block, suffix length 1..64, head dims of 64, 128 or 256, no NULL tensors
     fused = lambda T, dk, blk, ls, o_sfx=p: lib.fp_pop_fused_fwd(p, p, p, null, p, p, p, dec, p, o_sfx, null,
                                                                  1, T, 2, dk, 64, blk, ls, None)
     assert fused(100, 64, 64, 16) == -2 and b"multiple of block_size" in lib.fp_last_error()
     assert fused(128, 64, 64, 65) == -2 and b"suffix length" in lib.fp_last_error()
     assert fused(128, 64, 64, 0) == -2
-    assert fused(128, 256, 64, 16) == -3
+    assert fused(128, 96, 64, 16) == -3
     assert fused(128, 64, 64, 16, null) == -1
     assert lib.fp_pop_fused_bwd(p, p, p, null, p, p, p, dec, p, null, null, p, p, p, p, p, p, null,
                                 1, 128, 2, 64, 64, 64, 16, None) == -1

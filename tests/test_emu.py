@@ -74,6 +74,8 @@ FUSED_NAMES = ("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0")
     (2, 2, 80, 5, 1, 64, 128, None),     # block of a full and a short chunk, no initial state
     (1, 3, 24, 64, 1, 128, 64, 0.5),     # block shorter than a chunk, suffix as long as one
     (1, 1, 130, 1, 1, 64, 64, 0.0),      # one block of three chunks, one-token suffixes
+    (1, 2, 40, 9, 1, 256, 64, 0.5),      # two visits per chunk in the forward and dv passes
+    (1, 2, 64, 16, 1, 64, 256, 0.5),     # ... in the dq and dk passes
 ])
 def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std):
     decays = oracle.head_decays(H, (4, 9))

@@ -59,6 +59,8 @@ def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, ora
     (3, 5, 15, 7, 2, 64, 64),        # block and suffix shorter than a chunk
     (1, 2, 256, 64, 2, 128, 64),     # suffix as long as a chunk
     (2, 8, 32, 1, 2, 64, 128),       # one-token suffixes
+    (1, 3, 64, 16, 2, 256, 128),     # 256-wide keys: two visits per chunk in the forward and dv passes
+    (1, 2, 96, 24, 2, 128, 256),     # 256-wide values: two visits per chunk in the dq and dk passes
 ])
 def test_fused_parity_sweep(B, N, block, Ls, H, dk, dv):
     run_fused(B, N, block, Ls, H, dk, dv, 0.3, seed=N * block + Ls, decay_range=(5, 12))
