@@ -220,7 +220,6 @@ int backward(const Shape& s, const void* q, const void* k, const void* v, const 
 // is done only when the uncut call would leave at least two thirds of the compute units idle.
 int plan_segments(const Shape& s, int tiles) {
   constexpr int kMinChunks = 4;                 // shortest segment worth a workgroup of its own
-  if (s.dk > 128) return 1;                     // the state-only walk needs dA = dk of 64 or 128
   if (s.T % fpk::CH != 0) return 1;
   const int chunks = s.T / fpk::CH;
   const long long streams = (long long)s.B * s.H * tiles;

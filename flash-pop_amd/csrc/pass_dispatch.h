@@ -9,7 +9,7 @@
 namespace fpk {
 
 // Number of kernel instantiations `dispatch_pass` can pick from (its `slot` argument is below this).
-constexpr int PASS_KERNELS = 13;
+constexpr int PASS_KERNELS = 14;
 
 // Checks what the walks assume about `a` and chooses a.slots (workgroups per (head, column tile))
 // for a device with `compute_units` units.  Returns nullptr, or a message for the caller.
@@ -37,10 +37,10 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
     }
   }
   if (a.slots > a.B) a.slots = a.B;
-  if (a.state_only && (!narrow || blocks || suffix || !a.Rout))
-    return "state-only walk: needs dA of 64 or 128, a final-state buffer, no block states and no suffixes";
-  if (a.slots < a.B && (!narrow || blocks || suffix))
-    return "several batch entries per workgroup: only for the plain walk with dA of 64 or 128";
+  if (a.state_only && (blocks || suffix || !a.Rout))
+    return "state-only walk: needs a final-state buffer, no block states and no suffixes";
+  if (a.slots < a.B && ((!narrow && !a.state_only) || blocks || suffix))
+    return "several batch entries per workgroup: only for the state-only walk and the plain walk with dA of 64 or 128";
   return nullptr;
 }
 
@@ -99,6 +99,7 @@ int dispatch_pass(const PassArgs& a, Run&& run) {
   }
   // dA = 256: two visits per chunk, 128 of the 256 contraction columns each
   if (suffix) return run.template go<128, WALK_SUFFIX, 2>(12);
+  if (a.state_only) return run.template go<128, WALK_STATE, 2>(13);
   if (blocks) return run.template go<128, WALK_BLOCKS, 2>(10);
   return run.template go<128, WALK_PLAIN, 2>(11);
 }

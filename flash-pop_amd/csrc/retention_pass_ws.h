@@ -89,8 +89,7 @@ template <int DA, int MODE, int NH = 1>
 // else in `p` is common to all of them.
 FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char* lds, int wg, int nwg) {
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
-  static_assert(NH == 1 || (NH == 2 && (MODE == WALK_PLAIN || MODE == WALK_BLOCKS || MODE == WALK_SUFFIX)),
-                "two halves: plain, block and suffix walks only");
+  static_assert(NH == 1 || MODE != WALK_MULTI, "two halves: not with several sequences per workgroup and a read-out");
   constexpr bool STATE = MODE == WALK_STATE;
   constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI || STATE, SFX = MODE == WALK_SUFFIX;
   constexpr int X_LD = DA + 8;

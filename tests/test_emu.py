@@ -94,6 +94,7 @@ def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std):
     (1, 512, 1, 64, 64, 0.5, 2),       # the harness pretends to have 8 compute units: 1 stream -> 2 segments of 4 chunks
     (1, 1024, 1, 64, 128, None, 4),    # dk != dv, no initial state, 4 segments
     (1, 256, 1, 64, 64, 0.5, 1),       # too short to cut: same path as the plain entry point
+    (1, 512, 1, 256, 64, 0.5, 2),      # 256-wide keys: the state-only walk visits every chunk twice
 ])
 def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     decays = (0.97,) * H

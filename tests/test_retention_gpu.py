@@ -202,12 +202,13 @@ def test_decode_step_kernel_256_steps():
     hp.assert_close(s1, s1_ref, "state, no state")
 
 
-def test_split_entry_points_long_sequence_few_streams():
-    """fp_retention_*_split on a shape the library cuts into segments (4 streams on a 256-CU device):
-    against the oracle, against the unsplit entry points, and the workspace argument checks."""
+@pytest.mark.parametrize("B,T,H,dk,dv", [(1, 8192, 2, 128, 128), (1, 4096, 2, 256, 128)])
+def test_split_entry_points_long_sequence_few_streams(B, T, H, dk, dv):
+    """fp_retention_*_split on shapes the library cuts into segments (a few streams on a 256-CU device; with
+    256-wide keys the state-only walk visits every chunk twice): against the oracle, against the unsplit
+    entry points, and the workspace argument checks."""
     from flash_pop_amd import _lib
     lib = _lib.load()
-    B, T, H, dk, dv = 1, 8192, 2, 128, 128
     _say(f"[split] B{B} T{T} H{H} dk{dk} dv{dv}")
     decays = oracle.head_decays(H, (5, 9))
     q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=77, state_std=0.05, device=DEV)
