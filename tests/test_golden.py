@@ -94,3 +94,46 @@ def test_fused_pop_op_matches_golden(gold_fused):
     hp.assert_close(last, g["last"], "last", head_dim=1)
     for name, leaf in zip(FUSED_GRADS, leaves):
         hp.assert_close(leaf.grad, g[name], name, head_dim=1 if name == "ds0" else 2)
+
+
+LAYER_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layer_golden.npz")
+
+
+@pytest.fixture(scope="module")
+def gold_layer():
+    z = np.load(LAYER_PATH, allow_pickle=False)
+    return {k: torch.from_numpy(z[k]) for k in z.files}
+
+
+def test_layer_oracle_matches_golden(gold_layer):
+    g = gold_layer
+    T = g["q"].shape[1]
+    pos = g["start"][:, None] + torch.arange(T)[None]
+    for x, want, d_x, d_want in (("q", "q_rot", "d_q_rot", "dq"), ("k", "k_rot", "d_k_rot", "dk")):
+        assert torch.allclose(oracle.rotary(g[x], pos, g["theta"]), g[want], rtol=0, atol=2e-6), x
+        assert torch.allclose(oracle.rotary(g[d_x], pos, g["theta"], inverse=True), g[d_want], rtol=0, atol=2e-6), d_x
+    y = oracle.gated_group_norm(g["r"], g["gate"], float(g["eps"]))
+    assert torch.allclose(y, g["y"], rtol=1e-5, atol=1e-5)
+    d_r, d_gate = hp.oracle_gated_norm_grads(g["r"].to(hp.BF16), g["gate"].to(hp.BF16), g["d_out"].to(hp.BF16), float(g["eps"]))
+    hp.assert_close(d_r, g["d_r"], "d_r")
+    hp.assert_close(d_gate, g["d_gate"], "d_gate")
+
+
+@pytest.mark.gpu
+def test_layer_ops_match_golden(gold_layer):
+    from flash_pop_amd import XPos, gated_group_norm
+    g, dev = gold_layer, "cuda:0"
+    bf = lambda n: g[n].to(torch.bfloat16).to(dev)
+    q, k = bf("q").requires_grad_(), bf("k").requires_grad_()
+    xpos = XPos(q.shape[-1])
+    assert torch.equal(xpos.thetas, g["theta"])
+    rq, rk = xpos(q, k, g["start"].to(dev))
+    torch.autograd.backward([rq, rk], [bf("d_q_rot"), bf("d_k_rot")])
+    for got, want in ((rq, "q_rot"), (rk, "k_rot"), (q.grad, "dq"), (k.grad, "dk")):
+        hp.assert_close(got, g[want], want)
+    r, gate = bf("r").requires_grad_(), bf("gate").requires_grad_()
+    y = gated_group_norm(r, gate, float(g["eps"]))
+    y.backward(bf("d_out"))
+    hp.assert_close(y, g["y"], "y")
+    hp.assert_close(r.grad, g["d_r"], "d_r")
+    hp.assert_close(gate.grad, g["d_gate"], "d_gate")
