@@ -76,6 +76,21 @@ def gpu_leg(args):
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
     ms_per_step = wall * 1e3 / args.steps
 
+    # how fast the device streams a pass's tensors in this layout and access pattern with no staging and no math
+    lib = _lib.load()
+    y_probe = torch.empty_like(v)
+    probe = lambda: lib.fp_probe_stream_pattern(q.data_ptr(), k.data_ptr(), v.data_ptr(), y_probe.data_ptr(), B, T, H, dk, dv,
+                                                torch.cuda.current_stream().cuda_stream)
+    for _ in range(5):
+        probe()
+    pe = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    pe[0].record()
+    for _ in range(20):
+        probe()
+    pe[1].record()
+    torch.cuda.synchronize()
+    stream_ms = pe[0].elapsed_time(pe[1]) / 20
+
     f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
     b_fwd, b_bwd = algorithmic_bytes(B, T, H, dk, dv)
     tflops = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
@@ -120,6 +135,10 @@ def gpu_leg(args):
             # the forward launch on its own: one launch of retention_pass_ws_kernel<128, 0, 1>
             "forward_launch_ms": round(fwd_ms, 4),
             "forward_launch_algorithmic_gbs": round(b_fwd / (fwd_ms * 1e-3) / 1e9, 1),
+            # fp_probe_stream_pattern: the forward pass's loads and stores alone, same grid and placement
+            "stream_floor_ms": round(stream_ms, 4),
+            "stream_floor_gbs": round(b_fwd / (stream_ms * 1e-3) / 1e9, 1),
+            "forward_launch_vs_stream_floor": round(stream_ms / fwd_ms, 3),
         },
     }
 
@@ -358,6 +377,21 @@ def cpu_leg(sample_batch=8, reps=2):
         if i:
             times.append(time.perf_counter() - t0)
     sec = sorted(times)[len(times) // 2]
+    # how fast the device streams a pass's tensors in this layout and access pattern with no staging and no math
+    lib = _lib.load()
+    y_probe = torch.empty_like(v)
+    probe = lambda: lib.fp_probe_stream_pattern(q.data_ptr(), k.data_ptr(), v.data_ptr(), y_probe.data_ptr(), B, T, H, dk, dv,
+                                                torch.cuda.current_stream().cuda_stream)
+    for _ in range(5):
+        probe()
+    pe = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    pe[0].record()
+    for _ in range(20):
+        probe()
+    pe[1].record()
+    torch.cuda.synchronize()
+    stream_ms = pe[0].elapsed_time(pe[1]) / 20
+
     f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
     return {
         "value": round((f_fwd + f_bwd) / sec / 1e12, 4),

@@ -587,8 +587,22 @@ int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, voi
   return gated_norm(r, g, d_out, nullptr, d_r, d_g, rows, H, dv, eps, stream);
 }
 
+int fp_probe_stream_pattern(const void* x, const void* w, const void* z, void* y, int B, int T, int H, int dA, int dB,
+                            void* stream) {
+  if (!x || !w || !z || !y) return fail(FP_ERR_NULL_POINTER, "x, w, z and y must not be NULL");
+  if (B < 1 || H < 1 || T < fpk::CH || T % fpk::CH != 0)
+    return fail(FP_ERR_BAD_SHAPE, "B, H >= 1 and T a positive multiple of %d expected (got %d, %d, %d)", fpk::CH, B, H, T);
+  if (dA != 128 || dB < fpk::BV || dB % fpk::BV != 0)
+    return fail(FP_ERR_UNSUPPORTED_DIM, "the probe covers dA = 128 and dB a multiple of %d (got %d, %d)", fpk::BV, dA, dB);
+  if (misaligned(x) || misaligned(w) || misaligned(z) || misaligned(y)) return fail(FP_ERR_BAD_SHAPE, "tensors must be 16-byte aligned");
+  fpk::StreamProbeArgs a{in(x), in(w), in(z), out(y), B, T, H, dA, dB};
+  const char* msg = "";
+  if (fpk_launch_stream_probe(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s", msg);
+  return FP_OK;
+}
+
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1004; }
+int fp_version(void) { return 1005; }
 
 }  // extern "C"

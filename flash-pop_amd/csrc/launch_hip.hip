@@ -6,6 +6,7 @@
 #include "segment_scan.h"
 #include "decode_step.h"
 #include "layer_ops.h"
+#include "stream_probe.h"
 
 namespace {
 
@@ -49,6 +50,10 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_fwd_kernel(cons
 
 __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(const fpk::GatedNormArgs args) {
   fpk::gated_norm_bwd(args);
+}
+
+__global__ __launch_bounds__(fpk::PROBE_THREADS) void stream_probe_kernel(const fpk::StreamProbeArgs args) {
+  fpk::stream_probe(args, fpk::place_workgroup(fprt::block_index(), fprt::grid_size(), 1).wg);
 }
 
 // LDS above 64 KB has to be opted into once per device and kernel.  One bit per kernel (`slot`)
@@ -231,5 +236,16 @@ int fpk_launch_gated_norm(const fpk::GatedNormArgs& a, void* stream, const char*
   else
     hipLaunchKernelGGL(gated_norm_bwd_kernel, dim3((unsigned)blocks), dim3(fpk::LAYER_THREADS), 0,
                        static_cast<hipStream_t>(stream), a);
+  return launched(err);
+}
+
+int fpk_launch_stream_probe(const fpk::StreamProbeArgs& a, void* stream, const char** err) {
+  long long blocks = 0;
+  if (const char* why = fpk::plan_stream_probe(a, blocks)) {
+    *err = why;
+    return 1;
+  }
+  hipLaunchKernelGGL(stream_probe_kernel, dim3((unsigned)blocks), dim3(fpk::PROBE_THREADS), 0,
+                     static_cast<hipStream_t>(stream), a);
   return launched(err);
 }

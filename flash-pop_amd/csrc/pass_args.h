@@ -143,6 +143,15 @@ struct GatedNormArgs {
 };
 constexpr int LAYER_THREADS = 256;
 
+// The access pattern of one pass and nothing else (stream_probe.h): X, W [B,T,H,dA] read, the Z
+// tiles [B,T,H,dB] copied to Y.  T a multiple of 64, dA = 128, dB a multiple of 64.
+struct StreamProbeArgs {
+  const uint16_t *X, *W, *Z;
+  uint16_t* Y;
+  int B, T, H, dA, dB;
+};
+constexpr int PROBE_THREADS = 512;
+
 }  // namespace fpk
 
 // Launches the pass kernel on `stream` (a hipStream_t, or ignored by the CPU test harness).
@@ -168,3 +177,6 @@ int fpk_launch_decode(const fpk::DecodeArgs& args, void* stream, const char** er
 // Launch the rotary kernel / the gated per-head normalisation (forward if a.out, else backward).
 int fpk_launch_rotary(const fpk::RotaryArgs& args, void* stream, const char** err);
 int fpk_launch_gated_norm(const fpk::GatedNormArgs& args, void* stream, const char** err);
+
+// Launches the access-pattern probe (see stream_probe.h).  Same conventions as fpk_launch_pass.
+int fpk_launch_stream_probe(const fpk::StreamProbeArgs& args, void* stream, const char** err);

@@ -147,6 +147,14 @@ int fp_gated_group_norm_fwd(const void* r, const void* g, void* out, long long r
 int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, void* d_r, void* d_g, long long rows, int H,
                             int dv, double eps, void* stream);
 
+/* Measurement aid with no counterpart in the reference: streams the tensors of one pass in the
+ * pass kernel's access pattern (same grid, same workgroup placement, one chunk of loads in
+ * flight) without staging, barriers or arithmetic.  x, w [B,T,H,dA] are read, z [B,T,H,dB] is
+ * copied to y.  Its duration is the floor for a pass over these layouts; bench.py reports it
+ * beside the pass time.  T a multiple of 64, dA = 128, dB a multiple of 64. */
+int fp_probe_stream_pattern(const void* x, const void* w, const void* z, void* y, int B, int T, int H, int dA, int dB,
+                            void* stream);
+
 /* Message for the last nonzero return on this thread ("" if none). */
 const char* fp_last_error(void);
 

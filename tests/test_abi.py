@@ -31,7 +31,7 @@ def test_header_and_binding_agree(lib):
     assert names == sorted(_lib.SIGNATURES), (names, sorted(_lib.SIGNATURES))
     for n in names:
         assert hasattr(lib, n), f"{n} not exported"
-    assert lib.fp_version() == 1004
+    assert lib.fp_version() == 1005
 
 
 def test_argument_checks_return_codes(lib):
@@ -142,3 +142,12 @@ def test_layer_wrappers_refuse_cpu_tensors_and_bad_shapes():
         XPos(128)(q, q, 0)
     with pytest.raises(RuntimeError, match="GPU only"):
         gated_group_norm(q, q.flatten(-2))
+
+
+def test_stream_probe_checks_its_arguments(lib):
+    p, odd, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1008), None
+    assert lib.fp_probe_stream_pattern(p, p, null, p, 1, 64, 2, 128, 64, None) == -1
+    assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 100, 2, 128, 64, None) == -2
+    assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 64, 2, 64, 64, None) == -3
+    assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 64, 2, 128, 96, None) == -3
+    assert lib.fp_probe_stream_pattern(p, odd, p, p, 1, 64, 2, 128, 64, None) == -2

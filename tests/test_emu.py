@@ -184,3 +184,9 @@ def test_gated_group_norm(emu_lib, rows, H, dv):
     d_r_ref, d_g_ref = hp.oracle_gated_norm_grads(r, gate, d_out)
     hp.assert_close(d_r, d_r_ref, "d_r")
     hp.assert_close(d_g, d_g_ref, "d_g")
+
+
+def test_stream_probe_copies_z(emu_lib):
+    q, k, v, _ = hp.make_inputs(2, 128, 3, 128, 128, seed=12, state_std=None)
+    y = hp.raw_stream_probe(emu_lib, q, k, v)
+    assert torch.equal(y, v)
