@@ -377,21 +377,6 @@ def cpu_leg(sample_batch=8, reps=2):
         if i:
             times.append(time.perf_counter() - t0)
     sec = sorted(times)[len(times) // 2]
-    # how fast the device streams a pass's tensors in this layout and access pattern with no staging and no math
-    lib = _lib.load()
-    y_probe = torch.empty_like(v)
-    probe = lambda: lib.fp_probe_stream_pattern(q.data_ptr(), k.data_ptr(), v.data_ptr(), y_probe.data_ptr(), B, T, H, dk, dv,
-                                                torch.cuda.current_stream().cuda_stream)
-    for _ in range(5):
-        probe()
-    pe = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    pe[0].record()
-    for _ in range(20):
-        probe()
-    pe[1].record()
-    torch.cuda.synchronize()
-    stream_ms = pe[0].elapsed_time(pe[1]) / 20
-
     f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
     return {
         "value": round((f_fwd + f_bwd) / sec / 1e12, 4),
