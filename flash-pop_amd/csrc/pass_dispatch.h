@@ -52,9 +52,13 @@ struct WorkgroupId {
   int pass, wg;
 };
 FP_DEVICE WorkgroupId place_workgroup(int block, int nwg, int passes) {
-  if ((nwg & 7) != 0) return WorkgroupId{block % passes, block / passes};
-  const int xcd = block & 7, j = block >> 3;   // j-th workgroup that lands on this XCD
-  return WorkgroupId{j % passes, xcd * (nwg >> 3) + j / passes};
+  // XCD x runs the launch indices x, x + 8, ...; give it a contiguous range of the passes * nwg
+  // logical numbers (one more for the first `rem` XCDs when 8 does not divide the total), in
+  // which the passes of a workgroup and then the column tiles of a stream are neighbours.
+  const int total = nwg * passes, per = total >> 3, rem = total & 7;
+  const int xcd = block & 7, j = block >> 3;
+  const int logical = xcd * per + (xcd < rem ? xcd : rem) + j;
+  return WorkgroupId{logical % passes, logical / passes};
 }
 
 // Passes can share a launch if they walk the same shape in the same way (then they are the same
