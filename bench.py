@@ -117,6 +117,8 @@ def gpu_leg(args):
         "fwd_ms": round(fwd_ms, 4),
         "bwd_ms": round(bwd_ms, 4),
         "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        # the same time priced with only the causal half of every C x C tile counted (C -> (C + 1) / 2)
+        "tflops_causal_only": round(sum(algorithmic_flops(B, T, H, dk, dv, C=(CHUNK + 1) / 2)) / (ms_per_step * 1e-3) / 1e12, 2),
         "roofline": {
             "bound": "hbm",
             "kernel": "retention_pass_ws_kernel<128, 0, 1> (forward, dq) and retention_pass_multi_kernel<128, 0, 1> "
