@@ -42,6 +42,17 @@ FP_DEVICE float rsqrt_f32(float x) { return 1.0f / sqrtf(x); }
 // value held by lane (this lane ^ mask) of the wave; every lane of the wave has to call it
 FP_DEVICE float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
 
+// Transposing LDS read (ds_read_b64_tr_b16).  Every lane passes the address of four consecutive
+// 16-bit values; within each group of 16 lanes, lane i receives element i % 4 of the values read
+// by lanes 4 e + i / 4, e = 0..3.  With lane 4 r + q of a group pointing at columns 4 q .. 4 q + 3 of
+// row r of a row-major block of 4 rows x 16 columns, lane i gets column i of the four rows: an
+// MFMA operand that runs along the rows of a row-major tile.
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+FP_DEVICE u32x2 lds_read_tr16_b64(const uint16_t* p) {
+  return __builtin_bit_cast(
+      u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p)));
+}
+
 // Orders LDS traffic between the lanes of one wave.  The hardware executes a wave's LDS
 // instructions in order, so this only has to stop the compiler from reordering them.
 FP_DEVICE void wave_sync() { __builtin_amdgcn_wave_barrier(); }
@@ -76,10 +87,12 @@ FP_DEVICE int dbg_flags() { return 0; }
 #ifdef FPK_PROFILE
 __device__ unsigned long long* g_prof_buf = nullptr;
 FP_DEVICE void prof_stamp(int it, int slot) {
+  __builtin_amdgcn_sched_barrier(0);
   if (g_prof_buf && blockIdx.x == 0 && (threadIdx.x & 63) == 0 && it < 64) {
     const int wave = threadIdx.x >> 6;
     g_prof_buf[(wave * 64 + it) * 8 + slot] = __builtin_amdgcn_s_memtime();
   }
+  __builtin_amdgcn_sched_barrier(0);
 }
 #else
 FP_DEVICE void prof_stamp(int, int) {}

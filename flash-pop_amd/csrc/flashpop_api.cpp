@@ -26,6 +26,7 @@
 #include <cstdio>
 #include <cstring>
 #include <cstdint>
+#include <cstdlib>
 
 #include "pass_args.h"
 
@@ -172,9 +173,38 @@ int forward(const Shape& s, const void* q, const void* k, const void* v, const v
   return run(a, stream, "forward");
 }
 
+// The plain backward with dk = dv = 128 has a kernel of its own that reads q, k, v, dO once for dk
+// and dv together (retention_bwd_fused.h); it runs two workgroups per (batch, head) stream, so it
+// is chosen when those fill at least half of the device.  FLASHPOP_BWD=passes / fused in the
+// environment overrides the choice (for A/B measurements).
+bool use_fused_backward(const Shape& s, const void* d_blocks) {
+  if (s.dk != fpk::FB_D || s.dv != fpk::FB_D || d_blocks) return false;
+  if (const char* e = std::getenv("FLASHPOP_BWD")) {
+    if (std::strcmp(e, "passes") == 0) return false;
+    if (std::strcmp(e, "fused") == 0) return true;
+  }
+  return 4LL * s.B * s.H >= fpk_compute_units();
+}
+
+int backward_fused(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
+                   const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, void* stream) {
+  fpk::FusedBwdArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.q = in(q); a.k = in(k); a.v = in(v); a.dO = in(d_o);
+  a.dq = out(dq); a.dk = out(dk_); a.dv = out(dv_);
+  a.s0 = in(s0); a.ds_out = in(d_s_out); a.ds0 = out(d_s0);
+  a.B = s.B; a.T = s.T; a.H = s.H;
+  a.scale = 1.0f / std::sqrt((float)s.dk);
+  for (int h = 0; h < s.H; ++h) a.log2g[h] = (float)std::log2(decays[h]);
+  const char* msg = "";
+  if (fpk_launch_bwd_fused(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "fused backward: %s", msg);
+  return FP_OK;
+}
+
 int backward(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
              const void* d_o, const void* d_s_out, const void* d_blocks, int block, void* dq, void* dk_, void* dv_,
              void* d_s0, void* stream) {
+  if (use_fused_backward(s, d_blocks)) return backward_fused(s, q, k, v, s0, decays, d_o, d_s_out, dq, dk_, dv_, d_s0, stream);
   const float sc = 1.0f / std::sqrt((float)s.dk);
   const int nblk = block > 0 ? s.T / block : 0;
   fpk::PassArgs g, a;

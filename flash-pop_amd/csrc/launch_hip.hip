@@ -4,6 +4,7 @@
 #include "device_rt.h"
 #include "pass_dispatch.h"
 #include "segment_scan.h"
+#include "retention_bwd_fused.h"
 #include "decode_step.h"
 #include "layer_ops.h"
 #include "stream_probe.h"
@@ -29,6 +30,11 @@ __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_multi_kernel(
   const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, passes);
   const fpk::PassTensors io = id.pass == 0 ? fpk::tensors_of(first) : id.pass == 1 ? second : third;
   fpk::retention_pass_ws<DA, MODE, NH>(first, io, lds, id.wg, nwg);
+}
+
+__global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_kernel(const fpk::FusedBwdArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::fused_bwd(args, lds, fprt::block_index());
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -61,7 +67,7 @@ __global__ __launch_bounds__(fpk::PROBE_THREADS) void stream_probe_kernel(const 
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
-static_assert(2 * fpk::PASS_KERNELS <= 32, "one bit per kernel instantiation, single and paired");
+static_assert(2 * fpk::PASS_KERNELS <= 31, "one bit per kernel instantiation, single and paired");
 std::atomic<uint32_t> g_armed[kMaxDevices];
 
 template <typename Kernel, typename... More>
@@ -161,6 +167,38 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
     return 1;
   }
   return fpk::dispatch_pass(planned[0], DeviceMultiRun{planned, n, static_cast<hipStream_t>(stream), err});
+}
+
+int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* stream, const char** err) {
+  if (a.B < 1 || a.T < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || (long long)a.B * a.H * 2 > 0x7fffffffLL || !a.q || !a.k ||
+      !a.v || !a.dO || !a.dq || !a.dk || !a.dv) {
+    *err = "fused backward: bad arguments";
+    return 1;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    *err = "hipGetDevice failed";
+    return 1;
+  }
+  // the opt-in to more than 64 KB of LDS, once per device (bit 31 of the per-device word)
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1u << 31))) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(retention_bwd_fused_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, fpk::fb_lds_bytes()) != hipSuccess) {
+      (void)hipGetLastError();
+      *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
+      return 1;
+    }
+    if (tracked) g_armed[dev].fetch_or(1u << 31, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(retention_bwd_fused_kernel, dim3((unsigned)(2 * a.B * a.H)), dim3(fpk::FB_THREADS), fpk::fb_lds_bytes(),
+                     static_cast<hipStream_t>(stream), a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    *err = hipGetErrorString(e);
+    return 1;
+  }
+  return 0;
 }
 
 int fpk_launch_scan(const fpk::ScanArgs& a, void* stream, const char** err) {

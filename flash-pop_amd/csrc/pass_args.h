@@ -103,6 +103,20 @@ struct DecodeArgs {
   float scale;
   float gamma[MAX_HEADS];
 };
+// The fused backward for dk = dv = 128 (retention_bwd_fused.h): per (batch, head) stream one workgroup
+// walks backward for dk, dv and d_s0 and one walks forward for dq.
+constexpr int FB_D = 128;
+constexpr int FB_THREADS = 512;
+struct FusedBwdArgs {
+  const uint16_t *q, *k, *v, *dO;          // [B,T,H,128]
+  uint16_t *dq, *dk, *dv;
+  const uint16_t* s0;                      // [B,H,128,128], nullable (zeros)
+  const uint16_t* ds_out;                  // gradient of the final state, nullable (zeros)
+  uint16_t* ds0;                           // gradient of s0, nullable (not wanted)
+  int B, T, H;
+  float scale;                             // dk^-1/2
+  float log2g[MAX_HEADS];
+};
 constexpr int DECODE_THREADS = 256;
 constexpr int decode_lds_bytes(int dv) { return (DECODE_THREADS / (dv / 8)) * dv * 4; }
 
@@ -164,6 +178,9 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* stream, const char** err);
 // same rows in the same direction have the workgroups of a stream run side by side, so that those
 // rows come from HBM once.
 int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, const char** err);
+
+// Launches the fused backward (2 B H workgroups).  Same conventions as fpk_launch_pass.
+int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char** err);
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);

@@ -1,0 +1,671 @@
+// Fused retention backward for dk = dv = 128: two workgroups per (batch, head) stream, each
+// covering the full width of its tensors, in one launch.
+//
+//   "reverse" workgroup   walks the chunks from the last to the first and carries dS once.  It is
+//                         the dk pass and the dv pass of pass_args.h side by side:
+//                           pass 0 (dv):  X = k,  W = q,   Z = dO,  R = dS     (dk x dv)
+//                           pass 1 (dk):  X = v,  W = dO,  Z = q,   R = dS^T   (dv x dk)
+//                         W of one pass is Z of the other, so the state update
+//                         dS <- gamma^L dS + sum_j gamma^(j+1) q_j^T dO_j is done once and q, k, v,
+//                         dO are read once.
+//   "forward" workgroup   the dq pass (X = dO, W = v, Z = k, R = S^T), walking forward and
+//                         re-running the state recurrence from s0.
+//
+// Both kinds keep the four (three) 64 x 128 input tiles of a chunk row-major in LDS, single
+// buffered; the next chunk waits in registers.  Operands that run along the features of a tile are
+// 16-byte row reads, operands that run along its tokens come from the same tile through the
+// transposing LDS read, so no transposed copy is ever written.  Rows are padded to 136 elements
+// (68 banks): 16 consecutive rows of a row read, and the 4 rows r, r + 4, r + 8, r + 12 that the
+// lanes of a transposing read address, fall on different banks, and every address is a per-lane
+// base plus a compile-time offset.  Transposing reads therefore take the tokens of a k-step in a
+// strided order (below), which products with two such operands are free to do; score tiles are
+// computed with their rows permuted to match.
+//
+// Per chunk (reverse workgroup; the forward one is the same without the second pass):
+//   scores    three live 32 x 32 tiles per pass, one wave each, scaled by the decay, masked,
+//             rounded to bf16 and put into LDS in operand layout
+//   -- barrier --
+//   outputs   wave (pass, rt) owns rows 32 rt .. of Y^T for both 32-token halves:
+//             Y^T = wread (R^T X^T) + Z^T P^T, written to a staging tile
+//   update    wave w owns two 32 x 32 tiles of dS: decay, += (wkey W)^T Z
+//   -- barrier --
+//   the bf16 copy of dS, the next chunk's tiles and the staged outputs move
+//   -- barrier --
+#pragma once
+#include "pass_args.h"
+#include "lds_access.h"
+
+namespace fpk {
+
+constexpr int FB_LD = FB_D + 8;             // row pitch of every LDS tile, elements
+constexpr int FB_TILE = CH * FB_LD;        // elements of a 64 x 128 tile
+constexpr int FB_XP = 32 * 32;             // elements of one score tile in operand layout
+// reverse workgroup: q, k, v, dO tiles; bf16 copy of dS; two staging tiles; six score tiles
+constexpr int fb_lds_bytes() { return 2 * (4 * FB_TILE + FB_D * FB_LD + 2 * FB_TILE + 6 * FB_XP); }
+
+namespace fb {
+
+// element offset of (row, col) in a tile
+FP_DEVICE int at(int row, int col) { return row * FB_LD + col; }
+
+// Operand that runs along the columns of a tile: columns 16 t + 8 g .. + 7 of the lane's row.
+// `rowp` points at column 8 g of that row.
+FP_DEVICE u32x4 frag_cols(const uint16_t* rowp, int t) { return ld128(rowp + 16 * t); }
+
+// Operands that run along the rows (tokens) of a tile come from two transposing reads.  A lane
+// serves column cbase + lane % 32 and supplies the address of 4 columns of one row per read; the
+// rows that the four lanes 4 q + i of a group of 16 address become elements 0..3 of every lane
+// of the group.  Which rows of k-step t (rows 16 t .. 16 t + 15) a lane of half-wave g gets:
+//   TR_NAT  e < 4: 16 t + 2 g + 4 e,          e >= 4: 16 t + 2 g + 1 + 4 (e - 4)
+//           for products whose other operand is read the same way (any order serves)
+//   TR_ACC  e < 4: 16 t + g + 4 e,            e >= 4: 16 t + 2 + g + 4 (e - 4)
+//           the order in which a converted score tile (rows permuted by score_row) holds its tokens
+//   TR_SEQ  16 t + 8 g + e
+//           the order of a column-wise operand (rows four apart are what keeps the other two off
+//           the same banks; this one pays for consecutive rows)
+enum TrOrder { TR_NAT, TR_ACC, TR_SEQ };
+struct TrLane {
+  int lo, hi;   // element offsets of the two reads from (row 16 t, column cbase)
+};
+FP_DEVICE TrLane tr_lane(int lane, TrOrder order) {
+  const int g = lane >> 5, q = (lane & 15) >> 2;
+  const int col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int r_lo = order == TR_NAT ? 2 * g + 4 * q : order == TR_ACC ? g + 4 * q : 8 * g + q;
+  const int r_hi = order == TR_NAT ? r_lo + 1 : order == TR_ACC ? r_lo + 2 : r_lo + 4;
+  return TrLane{r_lo * FB_LD + col, r_hi * FB_LD + col};
+}
+// token (within its k-step) of element e of a TR_NAT operand
+FP_DEVICE int nat_token(int g, int e) { return 2 * g + 4 * (e & 3) + (e >> 2); }
+// row of the score tile that accumulator row m stands for: within each group of 16, m = 8 h + 4 g + e
+// holds token 4 e + 2 h + g, so that a TR_ACC operand meets the converted tile element for element
+FP_DEVICE int score_row(int m) { return (m & 16) + 4 * (m & 3) + 2 * ((m >> 3) & 1) + ((m >> 2) & 1); }
+
+FP_DEVICE u32x4 frag_rows(const uint16_t* tile, const TrLane& tl, int t, int cbase) {
+  const uint16_t* p = tile + 16 * t * FB_LD + cbase;
+  const u32x2 lo = fprt::lds_read_tr16_b64(p + tl.lo);
+  const u32x2 hi = fprt::lds_read_tr16_b64(p + tl.hi);
+  return u32x4{lo[0], lo[1], hi[0], hi[1]};
+}
+
+// eight packed bf16 times eight weights
+FP_DEVICE u32x4 weigh(u32x4 v, const float (&w)[8]) {
+  u32x4 o;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const float lo = __builtin_bit_cast(float, v[d] << 16) * w[2 * d];
+    const float hi = __builtin_bit_cast(float, v[d] & 0xffff0000u) * w[2 * d + 1];
+    o[d] = fprt::pack_bf16x2(lo, hi);
+  }
+  return o;
+}
+
+// What a workgroup of either kind shares: coordinates, the chunk feed and the output drain.
+struct Common {
+  int tid, wave, lane, g, c;
+  int b, h;
+  int T, nch;
+  uint32_t rowp;          // bytes between consecutive tokens of a tensor
+  float lg;
+  int ld_row, ld_piece;   // this thread's 16-byte pieces of a tile: rows ld_row and ld_row + 32
+};
+
+FP_DEVICE Common make_common(const FusedBwdArgs& p, int stream) {
+  Common k;
+  k.tid = fprt::thread_index();
+  k.wave = k.tid >> 6;
+  k.lane = k.tid & 63;
+  k.g = k.lane >> 5;
+  k.c = k.lane & 31;
+  k.h = stream % p.H;
+  k.b = stream / p.H;
+  k.T = p.T;
+  k.nch = (p.T + CH - 1) / CH;
+  k.rowp = (uint32_t)p.H * FB_D * 2;
+  k.lg = p.log2g[k.h];
+  k.ld_row = k.tid >> 4;
+  k.ld_piece = k.tid & 15;
+  return k;
+}
+
+// view of the rows of chunk `ci` of one tensor for this stream; rows past the sequence read as
+// zero and are dropped on stores
+FP_DEVICE fprt::BufView chunk_view(const Common& k, const void* base, int ci, bool store = false) {
+#ifdef FB_NOLOAD
+  if (!store) ci = -1;
+#endif
+#ifdef FB_NOSTORE
+  if (store) ci = -1;
+#endif
+  const bool ok = ci >= 0 && ci < k.nch;
+  const int t0 = ok ? ci * CH : 0;
+  const int L = ok ? (k.T - t0 < CH ? k.T - t0 : CH) : 0;
+  const char* ptr = static_cast<const char*>(base) + ((size_t)k.b * k.T + t0) * k.rowp + (size_t)k.h * FB_D * 2;
+  return fprt::make_buf(ptr, L > 0 ? (uint32_t)(L - 1) * k.rowp + FB_D * 2 : 0u);
+}
+
+template <int N>
+FP_DEVICE void load_tiles(const Common& k, const void* const (&src)[N], int ci, u32x4 (&pf)[2 * N]) {
+#pragma unroll
+  for (int x = 0; x < N; ++x) {
+    const fprt::BufView v = chunk_view(k, src[x], ci);
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      pf[2 * x + u] = fprt::buf_load128(v, (uint32_t)(k.ld_row + 32 * u) * k.rowp + k.ld_piece * 16);
+  }
+}
+template <int N>
+FP_DEVICE void stage_tiles(const Common& k, uint16_t* tiles, const u32x4 (&pf)[2 * N]) {
+#pragma unroll
+  for (int x = 0; x < N; ++x) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int row = k.ld_row + 32 * u;
+      st128(tiles + x * FB_TILE + at(row, 8 * k.ld_piece), pf[2 * x + u]);
+    }
+  }
+}
+// staging tile ([token][feature]) -> rows of chunk ci of `dst`
+FP_DEVICE void drain_tile(const Common& k, const uint16_t* tile, void* dst, int ci) {
+  const fprt::BufView v = chunk_view(k, dst, ci, true);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int row = k.ld_row + 32 * u;
+    fprt::buf_store128(v, (uint32_t)row * k.rowp + k.ld_piece * 16, ld128(tile + at(row, 8 * k.ld_piece)));
+  }
+}
+
+// 32 x 32 accumulator (rows n = nbase + acc_row(r, g), column token i) -> staging tile [i][n]
+FP_DEVICE void put_output(uint16_t* tile, int i, int nbase, int g, const f32x16& acc) {
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    u32x2 d;
+    d[0] = fprt::pack_bf16x2(acc[4 * qd], acc[4 * qd + 1]);
+    d[1] = fprt::pack_bf16x2(acc[4 * qd + 2], acc[4 * qd + 3]);
+    st64(tile + at(i, nbase + 8 * qd + 4 * g), d);
+  }
+}
+
+// The bf16 copy of a state matrix R (rows a = 0..127, columns n) lives in LDS as Rt[n][a].
+// accumulator tile (rows a = abase + acc_row, column n) -> Rt
+FP_DEVICE void put_state(uint16_t* Rt, int n, int abase, int g, const f32x16& acc) {
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    u32x2 d;
+    d[0] = fprt::pack_bf16x2(acc[4 * qd], acc[4 * qd + 1]);
+    d[1] = fprt::pack_bf16x2(acc[4 * qd + 2], acc[4 * qd + 3]);
+    st64(Rt + at(n, abase + 8 * qd + 4 * g), d);
+  }
+}
+FP_DEVICE f32x16 get_state(const uint16_t* Rt, int n, int abase, int g) {
+  f32x16 acc;
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    const u32x2 d = ld64(Rt + at(n, abase + 8 * qd + 4 * g));
+    acc[4 * qd] = __builtin_bit_cast(float, d[0] << 16);
+    acc[4 * qd + 1] = __builtin_bit_cast(float, d[0] & 0xffff0000u);
+    acc[4 * qd + 2] = __builtin_bit_cast(float, d[1] << 16);
+    acc[4 * qd + 3] = __builtin_bit_cast(float, d[1] & 0xffff0000u);
+  }
+  return acc;
+}
+// Global state matrix -> Rt, by all threads of the workgroup.  `along_a`: the matrix is stored
+// with a contiguous (element (a, n) at n * 128 + a), else with n contiguous (at a * 128 + n).
+FP_DEVICE void load_state(const Common& k, uint16_t* Rt, const uint16_t* src, bool along_a) {
+  const fprt::BufView v = fprt::make_buf(src, src ? (uint32_t)(FB_D * FB_D * 2) : 0u);   // null: zeros
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int pc = k.tid + FB_THREADS * u, major = pc >> 4, minor = (pc & 15) * 8;
+    const u32x4 d = fprt::buf_load128(v, (uint32_t)pc * 16);
+    if (along_a) {
+      st128(Rt + at(major, minor), d);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        reinterpret_cast<u16_m*>(Rt)[at(minor + e, major)] = (uint16_t)((e & 1) ? d[e >> 1] >> 16 : d[e >> 1] & 0xffffu);
+    }
+  }
+}
+FP_DEVICE void store_state(const Common& k, const uint16_t* Rt, uint16_t* dst, bool along_a) {
+  const fprt::BufView v = fprt::make_buf(dst, (uint32_t)(FB_D * FB_D * 2));
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int pc = k.tid + FB_THREADS * u, major = pc >> 4, minor = (pc & 15) * 8;
+    u32x4 d;
+    if (along_a) {
+      d = ld128(Rt + at(major, minor));
+    } else {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t lo = reinterpret_cast<const u16_m*>(Rt)[at(minor + 2 * w, major)];
+        const uint32_t hi = reinterpret_cast<const u16_m*>(Rt)[at(minor + 2 * w + 1, major)];
+        d[w] = lo | (hi << 16);
+      }
+    }
+    fprt::buf_store128(v, (uint32_t)pc * 16, d);
+  }
+}
+
+// One 32 x 32 score tile D[m][i] = sum_a W[j(m)][a] X[i][a] with j(m) = 32 jb + score_row(m) and
+// i = 32 ib + column.  `wrow`, `xrow`: this lane's rows of W and X at column 8 g.
+struct ScoreFrags {
+  u32x4 w[8], x[8];
+};
+FP_DEVICE void score_request(ScoreFrags& f, const uint16_t* wrow, const uint16_t* xrow, int t) {
+  f.w[t] = frag_cols(wrow, t);
+  f.x[t] = frag_cols(xrow, t);
+}
+// the products, then decay, mask, bf16, into `xp` in operand layout (two k-steps of 512 elements).
+// `mw`: decay weights of this lane's accumulator elements.  Element r stands for W token
+// score_const(r) + g and X token c; on the diagonal it is live if the W token is not before
+// (`reverse`) / not after the X token, and dead entries are cleared whatever the product was
+// (so that inf or nan from a masked token cannot leak).
+FP_DEVICE int score_const(int r) { return 16 * (r >> 3) + 4 * (r & 3) + 2 * ((r >> 2) & 1); }
+FP_DEVICE void score_finish(const f32x16& sc, const float (&mw)[16], bool diagonal, bool reverse, int c, int g,
+                            uint16_t* xp, int lane) {
+  const int x = reverse ? c - g : g - c;   // live: score_const(r) >= x (reverse) / -score_const(r) >= x
+  float v[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const bool live = !diagonal || (reverse ? score_const(r) >= x : -score_const(r) >= x);
+    v[r] = live ? sc[r] * mw[r] : 0.f;
+  }
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    u32x4 pm;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pm[e] = fprt::pack_bf16x2(v[8 * t + 2 * e], v[8 * t + 2 * e + 1]);
+    st128(xp + 512 * t + lane * 8, pm);
+  }
+}
+
+// Decay weights of this lane's accumulator elements of a score tile: s_intra gamma^distance, the
+// distance being |W token - X token| inside a diagonal tile (0 for dead entries) and 32 more in the
+// tile off the diagonal.
+FP_DEVICE void score_weights(float s_intra, float lg, bool diagonal, bool reverse, int c, int g, float (&mw)[16]) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int jl = score_const(r) + g;
+    const int d = reverse ? jl - c : c - jl;
+    mw[r] = s_intra * fprt::exp2_approx((float)(diagonal ? (d >= 0 ? d : 0) : 32 + d) * lg);
+  }
+}
+
+}  // namespace fb
+
+// ---------------------------------------------------------------------------------------------
+// reverse workgroup: dk, dv, d_s0
+// PASS: 0 for waves 0..3 (dv), 1 for waves 4..7 (dk); the two copies meet at the same barriers.
+template <int PASS>
+FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
+  using namespace fb;
+  const Common k = make_common(p, stream);
+  uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // tiles: 0 q, 1 k, 2 v, 3 dO
+  uint16_t* const Rt = TL + 4 * FB_TILE;                   // bf16(dS) as Rt[n = dv][a = dk]
+  uint16_t* const OUT = Rt + FB_D * FB_LD;                 // staging: 0 dv, 1 dk
+  uint16_t* const XP = OUT + 2 * FB_TILE;                  // score tiles [pass][tile][k-step][lane]
+  const uint16_t *Qs = TL, *Ks = TL + FB_TILE, *Vs = TL + 2 * FB_TILE, *Gs = TL + 3 * FB_TILE;
+
+  constexpr int pass = PASS;
+  const int rt = k.wave & 3, g = k.g, c = k.c, lane = k.lane;
+  const uint16_t* const Xs = pass ? Vs : Ks;
+  const uint16_t* const Ws = pass ? Gs : Qs;
+  const uint16_t* const Zs = pass ? Qs : Gs;
+  uint16_t* const out = OUT + pass * FB_TILE;
+  uint16_t* const xp_pass = XP + pass * 3 * FB_XP;
+  const float lg = k.lg;
+
+  // score tile of this wave (rt < 3): (jb, ib) = (0,0), (1,0), (1,1); live entries have j >= i
+  const int s_jb = rt == 0 ? 0 : 1, s_ib = rt == 2 ? 1 : 0;
+  float mw[16];
+  score_weights(p.scale, lg, s_jb == s_ib, true, c, g, mw);
+  const uint16_t* const s_wrow = Ws + at(32 * s_jb + score_row(c), 8 * g);
+  const uint16_t* const s_xrow = Xs + at(32 * s_ib + c, 8 * g);
+
+  const TrLane tr_acc = tr_lane(lane, TR_ACC), tr_nat = tr_lane(lane, TR_NAT), tr_seq = tr_lane(lane, TR_SEQ);
+  // state tiles of this wave: rows a = 32 at .., columns n = 32 (nt0 + {0, 1}) ..
+  const int at_ = k.wave & 3, nt0 = 2 * (k.wave >> 2);
+  // weights of the state update: wkey(j) = gamma^(j + 1) for the tokens of k-step 0
+  float wk0[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) wk0[e] = fprt::exp2_approx((float)(nat_token(g, e) + 1) * lg);
+  const float g16 = fprt::exp2_approx(16.f * lg);
+  // read-out weights of a full chunk and its decay
+  const float wread_full0 = p.scale * fprt::exp2_approx((float)(CH - 1 - c) * lg);
+  const float wread_full1 = p.scale * fprt::exp2_approx((float)(CH - 1 - 32 - c) * lg);
+  const float gL_full = fprt::exp2_approx((float)CH * lg);
+
+  const void* const src[4] = {p.q, p.k, p.v, p.dO};
+  u32x4 pf[8];
+  load_tiles<4>(k, src, k.nch - 1, pf);
+  load_state(k, Rt, p.ds_out ? p.ds_out + (size_t)stream * FB_D * FB_D : nullptr, false);
+  stage_tiles<4>(k, TL, pf);
+  load_tiles<4>(k, src, k.nch - 2, pf);
+  fprt::block_sync();
+  f32x16 racc[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) racc[u] = get_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g);
+
+  const uint16_t* const xrow0 = Xs + at(c, 8 * g);
+  const uint16_t* const xrow1 = Xs + at(32 + c, 8 * g);
+  const uint16_t* const rrow = Rt + at(32 * rt + c, 8 * g);
+
+  for (int ci = k.nch - 1; ci >= 0; --ci) {
+    const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
+    fprt::prof_stamp(k.nch - 1 - ci, 0);
+    // ---- what the previous chunk left to do: its outputs leave, the copy of its dS is written.
+    // Nothing reads either buffer before the next barrier.
+    if (ci < k.nch - 1) {
+      drain_tile(k, OUT, p.dv, ci + 1);
+      drain_tile(k, OUT + FB_TILE, p.dk, ci + 1);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
+    }
+    // ---- scores: the operands of a k-step are requested four k-steps ahead
+    if (rt < 3) {
+      ScoreFrags sf;
+      f32x16 sc = {0};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) score_request(sf, s_wrow, s_xrow, t);
+      fprt::sched_fence();
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        sc = fprt::mfma_32x32x16_bf16(sf.w[t], sf.x[t], sc);
+        if (t < 4) score_request(sf, s_wrow, s_xrow, t + 4);
+        fprt::sched_fence();
+      }
+      score_finish(sc, mw, s_jb == s_ib, true, c, g, xp_pass + rt * FB_XP, lane);
+    }
+    fprt::prof_stamp(k.nch - 1 - ci, 1);
+    // ---- state update, dS[a][n] = gamma^L dS + sum_j gamma^(j+1) q[j][a] dO[j][n], operands two
+    // k-steps ahead
+    u32x4 ua[4], ub0[4], ub1[4];
+    auto request_u = [&](int t) {
+      ua[t] = frag_rows(Qs, tr_nat, t, 32 * at_);
+      ub0[t] = frag_rows(Gs, tr_nat, t, 32 * nt0);
+      ub1[t] = frag_rows(Gs, tr_nat, t, 32 * (nt0 + 1));
+    };
+    request_u(0);
+    request_u(1);
+    const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) racc[u][r] *= gL;
+    }
+    float wk[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) wk[e] = wk0[e];
+    fprt::sched_fence();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const u32x4 wa = weigh(ua[t], wk);
+      racc[0] = fprt::mfma_32x32x16_bf16(wa, ub0[t], racc[0]);
+      racc[1] = fprt::mfma_32x32x16_bf16(wa, ub1[t], racc[1]);
+      if (t + 2 < 4) request_u(t + 2);
+      if (t < 3) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wk[e] *= g16;
+      }
+      fprt::sched_fence();
+    }
+    fprt::prof_stamp(k.nch - 1 - ci, 2);
+    fprt::block_sync();
+    fprt::prof_stamp(k.nch - 1 - ci, 3);
+
+    // ---- outputs: Y^T[n][i] = wread(i) sum_a R^T[n][a] X[i][a] + sum_j Z^T[n][j] P^T[j][i]
+    // operands of the read-out in two batches, the second requested before the first is used;
+    // the operands of the intra-chunk part follow while the read-out's products run
+    f32x16 acc[2];
+    acc[0] = f32x16{0};
+    acc[1] = f32x16{0};
+    // the operands of k-step t + 4 are requested when those of k-step t are used
+    u32x4 ra[8], x0[8], x1[8];
+    auto request = [&](int t) {
+      // pass 0: R^T = dS^T[n][a] is a row of Rt; pass 1: R^T = dS[a][n] runs along the rows of Rt
+      ra[t] = pass == 0 ? frag_cols(rrow, t) : frag_rows(Rt, tr_seq, t, 32 * rt);
+      x0[t] = frag_cols(xrow0, t);
+      x1[t] = frag_cols(xrow1, t);
+    };
+#pragma unroll
+    for (int t = 0; t < 4; ++t) request(t);
+    fprt::sched_fence();
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
+      acc[1] = fprt::mfma_32x32x16_bf16(ra[t], x1[t], acc[1]);
+      if (t + 4 < 8) request(t + 4);
+      fprt::sched_fence();
+    }
+    u32x4 za[4], pq0[4], pq1[2];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+      za[tj] = frag_rows(Zs, tr_acc, tj, 32 * rt);
+      pq0[tj] = ld128(xp_pass + (tj >> 1) * FB_XP + 512 * (tj & 1) + lane * 8);
+      if (tj >= 2) pq1[tj - 2] = ld128(xp_pass + 2 * FB_XP + 512 * (tj & 1) + lane * 8);
+    }
+    fprt::sched_fence();
+    fprt::prof_stamp(k.nch - 1 - ci, 4);
+    float wread0 = wread_full0, wread1 = wread_full1;
+    if (L != CH) {   // the last chunk of the sequence, visited first
+      const int e0 = L - 1 - c, e1 = L - 1 - 32 - c;
+      wread0 = p.scale * fprt::exp2_approx((float)(e0 > 0 ? e0 : 0) * lg);
+      wread1 = p.scale * fprt::exp2_approx((float)(e1 > 0 ? e1 : 0) * lg);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc[0][r] *= wread0;
+      acc[1][r] *= wread1;
+    }
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+      acc[0] = fprt::mfma_32x32x16_bf16(za[tj], pq0[tj], acc[0]);
+      if (tj >= 2) acc[1] = fprt::mfma_32x32x16_bf16(za[tj], pq1[tj - 2], acc[1]);
+    }
+    put_output(out, c, 32 * rt, g, acc[0]);
+    put_output(out, 32 + c, 32 * rt, g, acc[1]);
+    fprt::prof_stamp(k.nch - 1 - ci, 5);
+    fprt::block_sync();
+    fprt::prof_stamp(k.nch - 1 - ci, 6);
+
+    // ---- every read of this chunk's tiles is done: the next chunk's tiles take their place
+    stage_tiles<4>(k, TL, pf);
+    load_tiles<4>(k, src, ci - 2, pf);
+    fprt::prof_stamp(k.nch - 1 - ci, 7);
+    fprt::block_sync();
+  }
+  drain_tile(k, OUT, p.dv, 0);
+  drain_tile(k, OUT + FB_TILE, p.dk, 0);
+  if (p.ds0) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
+    fprt::block_sync();
+  }
+  if (p.ds0) store_state(k, Rt, p.ds0 + (size_t)stream * FB_D * FB_D, false);
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward workgroup: dq.  In pass notation X = dO, W = v, Z = k, R[a = dv][n = dk] = S^T.
+// Waves 0..3 ("output") own rows 32 w .. of Y^T = dq^T for both 32-token halves; waves 4..7
+// ("state") make the score tiles and own the four tiles of rows 32 (w - 4) .. of R.
+// STATE: the copy that waves 4..7 run; the two copies meet at the same barriers.
+template <bool STATE>
+FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
+  using namespace fb;
+  const Common k = make_common(p, stream);
+  uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // tiles: 0 X = dO, 1 W = v, 2 Z = k
+  uint16_t* const Rt = TL + 3 * FB_TILE;                   // bf16(R) as Rt[n][a]
+  uint16_t* const OUT = Rt + FB_D * FB_LD;
+  uint16_t* const XP = OUT + FB_TILE;                      // score tiles (0,0), (0,1), (1,1)
+  const uint16_t *Xs = TL, *Ws = TL + FB_TILE, *Zs = TL + 2 * FB_TILE;
+  const int g = k.g, c = k.c, lane = k.lane;
+  constexpr bool state_role = STATE;
+  const int rt = k.wave & 3;
+  const float lg = k.lg;
+
+  // score tile of state wave rt < 3: (jb, ib) = (0,0), (0,1), (1,1); live entries have i >= j
+  const int s_jb = rt == 2 ? 1 : 0, s_ib = rt == 0 ? 0 : 1;
+  float mw[16];
+  score_weights(p.scale, lg, s_jb == s_ib, false, c, g, mw);
+  const uint16_t* const s_wrow = Ws + at(32 * s_jb + score_row(c), 8 * g);
+  const uint16_t* const s_xrow = Xs + at(32 * s_ib + c, 8 * g);
+  const TrLane tr_acc = tr_lane(lane, TR_ACC), tr_nat = tr_lane(lane, TR_NAT);
+
+#ifdef FB_SEGREV
+  auto chunk_of = [&](int it) { const int seg = k.nch / FB_SEGREV - 1 - it / FB_SEGREV; return it < 0 || it >= k.nch ? -1 : seg * FB_SEGREV + it % FB_SEGREV; };
+#else
+  auto chunk_of = [&](int it) { return it; };
+#endif
+  const void* const src[3] = {p.dO, p.v, p.k};
+  u32x4 pf[6];
+  load_tiles<3>(k, src, chunk_of(0), pf);
+  // R[a][n] = S[n][a]: element (a, n) at n * 128 + a of s0
+  load_state(k, Rt, p.s0 ? p.s0 + (size_t)stream * FB_D * FB_D : nullptr, true);
+  stage_tiles<3>(k, TL, pf);
+  load_tiles<3>(k, src, chunk_of(1), pf);
+  fprt::block_sync();
+  f32x16 racc[4];
+  if constexpr (state_role) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) racc[u] = get_state(Rt, 32 * u + c, 32 * rt, g);
+  }
+  const uint16_t* const xrow0 = Xs + at(c, 8 * g);
+  const uint16_t* const xrow1 = Xs + at(32 + c, 8 * g);
+  const uint16_t* const rrow = Rt + at(32 * rt + c, 8 * g);
+  const float wread0 = fprt::exp2_approx((float)(c + 1) * lg), wread1 = fprt::exp2_approx((float)(32 + c + 1) * lg);
+  const float g16 = fprt::exp2_approx(16.f * lg);
+  const float gL_full = fprt::exp2_approx((float)CH * lg);
+  float wk_full[8];   // wkey of the tokens of the last k-step of a full chunk
+#pragma unroll
+  for (int e = 0; e < 8; ++e) wk_full[e] = p.scale * fprt::exp2_approx((float)(CH - 1 - (48 + nat_token(g, e))) * lg);
+
+  for (int it = 0; it < k.nch; ++it) {
+    const int ci = chunk_of(it);
+    const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
+    // what the previous chunk left to do (nothing reads either buffer before the next barrier)
+    if (it > 0) {
+      drain_tile(k, OUT, p.dq, chunk_of(it - 1));
+      if constexpr (state_role) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) put_state(Rt, 32 * u + c, 32 * rt, g, racc[u]);
+      }
+    }
+    if constexpr (state_role) {
+      if (rt < 3) {
+        ScoreFrags sf;
+        f32x16 sc = {0};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) score_request(sf, s_wrow, s_xrow, t);
+        fprt::sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          sc = fprt::mfma_32x32x16_bf16(sf.w[t], sf.x[t], sc);
+          if (t < 4) score_request(sf, s_wrow, s_xrow, t + 4);
+          fprt::sched_fence();
+        }
+        score_finish(sc, mw, s_jb == s_ib, false, c, g, XP + rt * FB_XP, lane);
+      }
+      // R[a][n] = gamma^L R + sum_j s gamma^(L-1-j) W[j][a] Z[j][n]
+      const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) racc[u][r] *= gL;
+      }
+      // wkey(j) = s gamma^(L-1-j).  Full chunk: the last k-step's weights, times gamma^16 per
+      // earlier k-step.  Short chunk (the last one of a sequence): exponents clamped at 0 one by
+      // one (those rows are zero, the weight only has to stay finite).
+      float w[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w[e] = wk_full[e];
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        const int t = 3 - tt;
+        if (L != CH) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int x = L - 1 - (16 * t + nat_token(g, e));
+            w[e] = p.scale * fprt::exp2_approx((float)(x > 0 ? x : 0) * lg);
+          }
+        }
+        u32x4 ub[4];
+        const u32x4 ua = frag_rows(Ws, tr_nat, t, 32 * rt);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) ub[u] = frag_rows(Zs, tr_nat, t, 32 * u);
+        const u32x4 wa = weigh(ua, w);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) racc[u] = fprt::mfma_32x32x16_bf16(wa, ub[u], racc[u]);
+        if (tt < 3) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e] *= g16;
+        }
+      }
+    }
+    fprt::block_sync();
+
+    if constexpr (!state_role) {
+      // Y^T[n][i] = gamma^(i+1) sum_a R^T[n][a] X[i][a] + sum_j Z^T[n][j] P^T[j][i]
+      f32x16 acc[2];
+      acc[0] = f32x16{0};
+      acc[1] = f32x16{0};
+      u32x4 ra[8], x0[8], x1[8];
+      auto request = [&](int t) {
+        ra[t] = frag_cols(rrow, t);
+        x0[t] = frag_cols(xrow0, t);
+        x1[t] = frag_cols(xrow1, t);
+      };
+#pragma unroll
+      for (int t = 0; t < 4; ++t) request(t);
+      fprt::sched_fence();
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
+        acc[1] = fprt::mfma_32x32x16_bf16(ra[t], x1[t], acc[1]);
+        if (t + 4 < 8) request(t + 4);
+        fprt::sched_fence();
+      }
+      // tokens j < 32 reach both halves (tiles (0,0), (0,1)), the others only the second
+      u32x4 za[4], pq1[4], pq0[2];
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        za[tj] = frag_rows(Zs, tr_acc, tj, 32 * rt);
+        pq1[tj] = ld128(XP + (tj < 2 ? 1 : 2) * FB_XP + 512 * (tj & 1) + lane * 8);
+        if (tj < 2) pq0[tj] = ld128(XP + 512 * (tj & 1) + lane * 8);
+      }
+      fprt::sched_fence();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[0][r] *= wread0;
+        acc[1][r] *= wread1;
+      }
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        acc[1] = fprt::mfma_32x32x16_bf16(za[tj], pq1[tj], acc[1]);
+        if (tj < 2) acc[0] = fprt::mfma_32x32x16_bf16(za[tj], pq0[tj], acc[0]);
+      }
+      put_output(OUT, c, 32 * rt, g, acc[0]);
+      put_output(OUT, 32 + c, 32 * rt, g, acc[1]);
+    }
+    fprt::block_sync();
+
+    stage_tiles<3>(k, TL, pf);
+    load_tiles<3>(k, src, chunk_of(it + 2), pf);
+    fprt::block_sync();
+  }
+  drain_tile(k, OUT, p.dq, chunk_of(k.nch - 1));
+}
+
+// launch index -> kind and stream: the reverse workgroups (the longer ones) come first
+FP_DEVICE void fused_bwd(const FusedBwdArgs& p, char* lds, int block) {
+  const int streams = p.B * p.H;
+#ifdef FB_ONLY
+  if ((block < streams) != (FB_ONLY == 0)) return;
+#endif
+  if (block < streams) {
+    if (fprt::thread_index() < 256) fused_bwd_reverse<0>(p, lds, block);
+    else fused_bwd_reverse<1>(p, lds, block);
+  }
+  else if (fprt::thread_index() < 256) fused_bwd_forward<false>(p, lds, block - streams);
+  else fused_bwd_forward<true>(p, lds, block - streams);
+}
+
+}  // namespace fpk

@@ -21,6 +21,7 @@ struct WaveShared {
   uint16_t A[64][8];
   uint16_t Bm[64][8];
   float xchg[64];
+  uint16_t tr[64][4];
   pthread_barrier_t bar;
 };
 
@@ -90,6 +91,22 @@ FP_DEVICE float lane_xor(float v, int mask) {
   const float r = g_lane.wave->xchg[lane ^ mask];
   wave_sync();
   return r;
+}
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element i % 4 of the four
+// values read by lanes 4 e + i / 4, e = 0..3
+FP_DEVICE u32x2 lds_read_tr16_b64(const uint16_t* p) {
+  WaveShared* w = g_lane.wave;
+  const int lane = g_lane.tid & 63;
+  std::memcpy(w->tr[lane], p, 8);
+  wave_sync();
+  const int grp = lane & ~15, i = lane & 15;
+  uint16_t out[4];
+  for (int e = 0; e < 4; ++e) out[e] = w->tr[grp + 4 * e + i / 4][i % 4];
+  wave_sync();
+  u32x2 v;
+  std::memcpy(&v, out, 8);
+  return v;
 }
 
 FP_DEVICE int dbg_flags() { return 0; }

@@ -3,6 +3,7 @@
 #include "device_rt.h"
 #include "pass_dispatch.h"
 #include "segment_scan.h"
+#include "retention_bwd_fused.h"
 #include "decode_step.h"
 #include "layer_ops.h"
 #include "stream_probe.h"
@@ -98,6 +99,14 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
 // Pretends the chip has 8 compute units, so that small test shapes take the paths that large
 // ones take on a real device (several sequences per workgroup, split sequences).
 int fpk_compute_units() { return 8; }
+
+int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* /*stream*/, const char** err) {
+  if (a.B < 1 || a.T < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || !a.q || !a.k || !a.v || !a.dO || !a.dq || !a.dk || !a.dv) {
+    *err = "fused backward: bad arguments";
+    return 1;
+  }
+  return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(), [&](char* l) { fpk::fused_bwd(a, l, fprt::block_index()); });
+}
 
 int fpk_launch_scan(const fpk::ScanArgs& a, void* /*stream*/, const char** err) {
   if (a.M % fpk::SCAN_VEC != 0 || a.B < 1 || a.S < 1 || a.H < 1 || !a.U || !a.init) {
