@@ -39,8 +39,9 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
   if (a.slots > a.B) a.slots = a.B;
   if (a.state_only && (blocks || suffix || !a.Rout))
     return "state-only walk: needs a final-state buffer, no block states and no suffixes";
-  if (a.slots < a.B && ((!narrow && !a.state_only) || blocks || suffix))
-    return "several batch entries per workgroup: only for the state-only walk and the plain walk with dA of 64 or 128";
+  // (with two visits per chunk only the first half of the state is handed over between sequences)
+  if (a.slots < a.B && (!narrow || blocks || suffix))
+    return "several batch entries per workgroup: only for the plain and state-only walks with dA of 64 or 128";
   return nullptr;
 }
 

@@ -14,6 +14,16 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+def refuse_capture(what):
+    """The pass kernels must not be recorded into a HIP graph: instantiating a graph that holds
+    them has crashed the host process (a segmentation fault inside the runtime, after every
+    launch had been recorded without error).  Until that is understood the ops raise instead."""
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(
+            f"{what} cannot be captured into a HIP graph with this ROCm / PyTorch build "
+            "(graph instantiation crashes the process); call it eagerly, outside torch.cuda.graph")
+
+
 def prepare(q, k, v, s, head_decays):
     """Validate like the reference's asserts (fused_retention/__init__.py:20,
     pop_retention/__init__.py:17-18) and return contiguous tensors plus the shape."""
@@ -45,6 +55,7 @@ def _workspace(lib, shape, device):
 
 
 def retention_fwd(q, k, v, s, decays, shape):
+    refuse_capture("retention_fwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
     o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
@@ -62,6 +73,7 @@ def retention_fwd(q, k, v, s, decays, shape):
 
 
 def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
+    refuse_capture("pop_retention_fwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
     o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
@@ -75,6 +87,7 @@ def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
 
 def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0):
     """Gradients for both ops; block_size is None for the plain op."""
+    refuse_capture("retention_bwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
     d_o = d_o.contiguous()
@@ -120,6 +133,7 @@ def prepare_suffixes(q_sfx, k_sfx, v_sfx, shape, block_size):
 
 
 def pop_fused_fwd(q, k, v, s, sfx, decays, block_size, shape):
+    refuse_capture("pop_fused_fwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
     o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
@@ -134,6 +148,7 @@ def pop_fused_fwd(q, k, v, s, sfx, decays, block_size, shape):
 
 
 def pop_fused_bwd(q, k, v, s, sfx, decays, block_size, shape, d_o, d_o_sfx, d_s_out, want_ds0):
+    refuse_capture("pop_fused_bwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
     d_o, d_o_sfx = d_o.contiguous(), d_o_sfx.contiguous()

@@ -151,3 +151,27 @@ def test_stream_probe_checks_its_arguments(lib):
     assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 64, 2, 64, 64, None) == -3
     assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 64, 2, 128, 96, None) == -3
     assert lib.fp_probe_stream_pattern(p, odd, p, p, 1, 64, 2, 128, 64, None) == -2
+
+
+def test_pass_ops_refuse_graph_capture(monkeypatch):
+    """Capturing the pass kernels into a HIP graph has crashed the host process, so the Python
+    ops raise while the current stream is capturing.  The flag is mocked: no GPU is touched."""
+    import torch
+    from flash_pop_amd import _ops
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: True)
+    q = torch.zeros(1, 4, 1, 64, dtype=torch.bfloat16)
+    sfx = (q, q, q)
+    calls = [
+        lambda: _ops.retention_fwd(q, q, q, None, (0.9,), (1, 4, 1, 64, 64)),
+        lambda: _ops.pop_retention_fwd(q, q, q, None, (0.9,), 2, (1, 4, 1, 64, 64)),
+        lambda: _ops.retention_bwd(q, q, q, None, (0.9,), (1, 4, 1, 64, 64), q, None, None, None, False),
+        lambda: _ops.pop_fused_fwd(q, q, q, None, sfx, (0.9,), 2, (1, 4, 1, 64, 64)),
+        lambda: _ops.pop_fused_bwd(q, q, q, None, sfx, (0.9,), 2, (1, 4, 1, 64, 64), q, q, None, False),
+    ]
+    for call in calls:
+        with pytest.raises(RuntimeError, match="cannot be captured into a HIP graph"):
+            call()
+    # the small kernels (decode step, rotary, gated norm) stay capturable: no guard in their wrappers
+    import inspect
+    for name in ("decode_step", "rotary_qk", "gated_norm_fwd", "gated_norm_bwd"):
+        assert "refuse_capture" not in inspect.getsource(getattr(_ops, name))

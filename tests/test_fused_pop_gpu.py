@@ -16,7 +16,8 @@ def _say(msg):
     print(msg, flush=True)
 
 
-def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, oracle_batches=None, d_last=True):
+def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, oracle_batches=None, d_last=True,
+              oracle_device="cpu", literal=None):
     from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
     T = N * block
     _say(f"[fused pop] B{B} N{N} block{block} Ls{Ls} H{H} dk{dk} dv{dv} s0={state_std} seed={seed}")
@@ -40,16 +41,18 @@ def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, ora
         cut = lambda t, w: None if t is None else t[w]
         o_ref, os_ref, last_ref, g_ref = hp.oracle_fused(
             q[sl], k[sl], v[sl], cut(s, sl), [t[ssl] for t in sfx], decays, block,
-            (cot[0][sl], cot[1][ssl], cut(cot[2], sl)))
-        hp.assert_close(o[sl], o_ref, f"o[b={b}]", head_dim=2)
-        hp.assert_close(o_sfx[ssl], os_ref, f"o_sfx[b={b}]", head_dim=2)
-        hp.assert_close(last[sl], last_ref, f"last_state[b={b}]", head_dim=1)
+            (cot[0][sl], cot[1][ssl], cut(cot[2], sl)), device=oracle_device)
+        pairs = [(f"o[b={b}]", o[sl], o_ref, 2), (f"o_sfx[b={b}]", o_sfx[ssl], os_ref, 2), (f"last S[b={b}]", last[sl], last_ref, 1)]
         leaves = ctx[:3] + sx + [ctx[3]]
         for name, leaf, ref in zip(GRADS, leaves, g_ref):
             if ref is None:
                 continue
             w = sl if "sfx" not in name else ssl
-            hp.assert_close(leaf.grad[w], ref, f"{name}[b={b}]", head_dim=1 if name == "ds0" else 2)
+            pairs.append((f"{name}[b={b}]", leaf.grad[w], ref, 1 if name == "ds0" else 2))
+        for name, got, ref, head_dim in pairs:
+            hp.assert_close(got, ref, name, head_dim=head_dim)
+            if literal is not None:
+                hp.check_literal(got, ref, name, literal)
     return o, o_sfx, last
 
 
@@ -123,5 +126,30 @@ def test_fused_argument_errors():
 
 def test_config4_fused():
     """Benchmark configuration 4 in one walk: B8 H16 d128, T4096 in 64-token blocks, 65 suffixes of 16 tokens
-    per sequence.  Oracle on one sequence."""
-    run_fused(8, 64, 64, 16, 16, 128, 128, 0.05, seed=40, oracle_batches=[5])
+    per sequence.  Every sequence against the oracle, which runs on the GPU."""
+    run_fused(8, 64, 64, 16, 16, 128, 128, 0.05, seed=40, oracle_device=DEV, literal={})
+
+
+def test_config5_layer_shapes_fused_pop_and_decode():
+    """The retention shapes of benchmark configuration 5 (B8, 12 heads, dk 64, dv 128, T2048 in
+    64-token blocks with 16-token suffixes): the fused POP op with all gradients against the oracle
+    on every sequence, then 256 recurrent decode steps from its last state against the oracle's
+    recurrent step (state rounded to bf16 after every step, as the kernel stores it)."""
+    from flash_pop_amd import retention_recurrent
+    B, H, dk, dv = 8, 12, 64, 128
+    o, o_sfx, last = run_fused(B, 32, 64, 16, H, dk, dv, 0.05, seed=50, oracle_device=DEV, literal={})
+    decays = oracle.head_decays(H)
+    q, k, v, _ = hp.make_inputs(B, 256, H, dk, dv, seed=51)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    state = last.detach().clone()
+    ref_state = last.detach().float()
+    outs, refs = [], []
+    for t in range(256):
+        o_t, state = retention_recurrent(qd[:, t], kd[:, t], vd[:, t], decays, state, in_place=True)
+        outs.append(o_t)
+        r_t, ref_state = oracle.recurrent_step(qd[:, t].float(), kd[:, t].float(), vd[:, t].float(), ref_state, decays)
+        ref_state = ref_state.to(hp.BF16).float()
+        refs.append(r_t)
+    torch.cuda.synchronize()
+    hp.assert_close(torch.stack(outs, 1), torch.stack(refs, 1), "decode o", head_dim=2)
+    hp.assert_close(state, ref_state, "decode state", head_dim=1)

@@ -71,7 +71,7 @@ def test_pop_outputs_equal_plain_outputs():
     assert torch.equal(o_pop, o) and torch.equal(states[:, -1], S)
 
 
-def _suffix_case(B, N, block, Ls, H, dk, dv, seed, oracle_batches):
+def _suffix_case(B, N, block, Ls, H, dk, dv, seed, oracle_batches, oracle_device="cpu", literal=None):
     """Context through flash_pop_retention, N + 1 suffixes per sequence through
     fused_chunk_retention started from [S0, block states] (flash_pop/pop_retnet.py:152-171),
     gradients chained through both ops by autograd."""
@@ -92,18 +92,21 @@ def _suffix_case(B, N, block, Ls, H, dk, dv, seed, oracle_batches):
 
     for b in oracle_batches:
         sl, ssl = slice(b, b + 1), slice(b * (N + 1), (b + 1) * (N + 1))
-        ins = [t[sl].float().requires_grad_() for t in (q, k, v, s)]
-        sins = [t[ssl].float().requires_grad_() for t in (qs, ks, vs)]
+        ins = [t[sl].to(oracle_device).float().requires_grad_() for t in (q, k, v, s)]
+        sins = [t[ssl].to(oracle_device).float().requires_grad_() for t in (qs, ks, vs)]
         o_ref, st_ref = oracle.pop_retention(*ins, decays, block)
         os_ref = oracle.pop_suffix_retention(*sins, ins[3], st_ref, decays)
-        loss = (o_ref * d_o[sl].float()).sum() + (os_ref * d_os[ssl].float()).sum()
+        loss = (o_ref * d_o[sl].to(oracle_device).float()).sum() + (os_ref * d_os[ssl].to(oracle_device).float()).sum()
         grads = torch.autograd.grad(loss, ins + sins)
-        hp.assert_close(o[sl], o_ref.detach(), "ctx o", head_dim=2)
-        hp.assert_close(o_sfx[ssl], os_ref.detach(), "suffix o", head_dim=2)
+        pairs = [(f"ctx o[b={b}]", o[sl], o_ref.detach(), 2), (f"suffix o[b={b}]", o_sfx[ssl], os_ref.detach(), 2)]
         for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), ctx_leaves, grads[:4]):
-            hp.assert_close(leaf.grad[sl], ref, f"ctx {name}", head_dim=1 if name == "ds0" else 2)
+            pairs.append((f"ctx {name}[b={b}]", leaf.grad[sl], ref, 1 if name == "ds0" else 2))
         for name, leaf, ref in zip(("dq", "dk", "dv"), sfx_leaves, grads[4:]):
-            hp.assert_close(leaf.grad[ssl], ref, f"suffix {name}", head_dim=2)
+            pairs.append((f"suffix {name}[b={b}]", leaf.grad[ssl], ref, 2))
+        for name, got, ref, head_dim in pairs:
+            hp.assert_close(got, ref, name, head_dim=head_dim)
+            if literal is not None:
+                hp.check_literal(got, ref, name, literal)
 
 
 def test_pop_suffix_path_small():
@@ -112,5 +115,6 @@ def test_pop_suffix_path_small():
 
 def test_config4_pop_with_suffixes():
     """Benchmark configuration 4: B8 H16 d128, T4096 in 64-token blocks, 16-token suffixes at every boundary
-    (N + 1 = 65 per sequence, the first from S0).  Oracle on one sequence."""
-    _suffix_case(B=8, N=64, block=64, Ls=16, H=16, dk=128, dv=128, seed=40, oracle_batches=[5])
+    (N + 1 = 65 per sequence, the first from S0).  Every sequence against the oracle, which runs on the GPU."""
+    _suffix_case(B=8, N=64, block=64, Ls=16, H=16, dk=128, dv=128, seed=40, oracle_batches=range(8), oracle_device=DEV,
+                 literal={})
