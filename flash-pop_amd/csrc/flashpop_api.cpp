@@ -483,6 +483,28 @@ int fp_retention_fwd_split(const void* q, const void* k, const void* v, const vo
   return forward_split(s, segments, q, k, v, s0, head_decays, o, s_out, workspace, stream);
 }
 
+int fp_retention_fwd_split_static(const void* q, const void* k, const void* v, const void* s0,
+                                  const double* head_decays, void* o, void* s_out, int B, int T, int H, int dk, int dv,
+                                  void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
+  const int segments = plan_forward(s);
+  if (segments <= 1) return forward(s, q, k, v, s0, head_decays, o, s_out, nullptr, 0, stream);
+  const size_t need = workspace_bytes(s, segments);
+  if (need > fpk::STATIC_SCRATCH_BYTES)
+    return fail(FP_ERR_BAD_SHAPE,
+                "this shape needs %zu bytes of segment states, more than the %zu bytes of the library's own scratch: "
+                "use fp_retention_fwd_split with a workspace",
+                need, (size_t)fpk::STATIC_SCRATCH_BYTES);
+  void* scratch_ptr = nullptr;
+  const char* msg = "";
+  if (fpk_static_scratch(&scratch_ptr, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s", msg);
+  // nothing in the scratch has to start at zero: the state-only pass writes every segment's
+  // contribution and the scan every starting state before anything reads them
+  return forward_split(s, segments, q, k, v, s0, head_decays, o, s_out, scratch_ptr, stream);
+}
+
 int fp_retention_bwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
                            const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B,
                            int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes_given, void* stream) {

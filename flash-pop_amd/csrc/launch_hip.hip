@@ -111,6 +111,43 @@ extern "C" int fpk_dbg_set(int flags) {
 }
 #endif
 
+// ---- scratch memory that no call allocates ------------------------------------------------------
+// fp_retention_fwd_split_static runs the split-sequence forward without a workspace from the
+// caller: the segment states live in this array, of which every device holds its own copy at
+// its own address from the moment the code object is loaded until the process ends.  The name of
+// the array means nothing to host code; its address on the current device comes from
+// hipGetSymbolAddress, once per device, and is what kernels and host calls are given afterwards.
+static __device__ __align__(256) unsigned char scratch[fpk::STATIC_SCRATCH_BYTES];
+
+namespace {
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+}
+
+int fpk_static_scratch(void** ptr, const char** err) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    *err = "hipGetDevice failed";
+    return 1;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    *err = "device index beyond the table of per-device scratch addresses";
+    return 1;
+  }
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    // first call on this device (it is the current one): look the array's address up and keep it
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      *err = "hipGetSymbolAddress(scratch) failed";
+      return 1;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return 0;
+}
+
 // Compute units of the current device (cached per thread and device).
 int fpk_compute_units() {
   static thread_local int dev_cached = -1, cus = 0;

@@ -16,6 +16,7 @@
 // passes are four choices of (X, W, Z, R); see flashpop_api.cpp.
 #pragma once
 #include <stdint.h>
+#include <stddef.h>
 
 namespace fpk {
 
@@ -184,6 +185,14 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);
+
+// Bytes of the library's own scratch array (one per device, see fpk_static_scratch).
+namespace fpk {
+constexpr size_t STATIC_SCRATCH_BYTES = 8u << 20;
+}
+// Address of the scratch array on the current device (device memory, 256-byte aligned,
+// fpk::STATIC_SCRATCH_BYTES long); looked up on the first call on each device, never allocated.
+int fpk_static_scratch(void** ptr, const char** err);
 
 // Compute units of the current device (what the launcher sizes its grids against).
 int fpk_compute_units();

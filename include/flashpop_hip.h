@@ -72,6 +72,20 @@ int fp_retention_bwd_split(const void* q, const void* k, const void* v, const vo
                            const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B,
                            int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes, void* stream);
 
+/* fp_retention_fwd_split without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory at the call:
+ * code under HIP graph capture set-up, tight serving loops, harnesses that forbid hipMalloc.  The
+ * segment states live in an array inside the library's code object (8 MiB per device, held from
+ * the first use of the library on that device until the process ends).  Same results as
+ * fp_retention_fwd_split, bit for bit.  A shape whose segment states need more than 8 MiB
+ * (fp_retention_workspace_bytes says how much; on a 256-CU device only dk = 256 can) is rejected
+ * with FP_ERR_BAD_SHAPE.  Every call on
+ * a device uses that device's one array: two calls that overlap in time on one device (different
+ * streams or threads) race; calls on one stream are ordered and safe. */
+int fp_retention_fwd_split_static(const void* q, const void* k, const void* v, const void* s0,
+                                  const double* head_decays, void* o, void* s_out, int B, int T, int H, int dk, int dv,
+                                  void* stream);
+
 /* Replaces the kernel call in FlashPOPRetention.forward
  * (flash_pop/pop_retention/__init__.py:14-31).
  *   block_states  out: state after every FULL block of block_size tokens,

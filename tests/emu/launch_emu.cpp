@@ -96,6 +96,13 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
   return fpk::dispatch_pass(planned[0], HarnessMultiRun{planned, n});
 }
 
+// the harness's stand-in for the library's own scratch array (host memory here)
+int fpk_static_scratch(void** ptr, const char** /*err*/) {
+  static std::vector<unsigned char> scratch(fpk::STATIC_SCRATCH_BYTES);
+  *ptr = scratch.data();
+  return 0;
+}
+
 // Pretends the chip has 8 compute units, so that small test shapes take the paths that large
 // ones take on a real device (several sequences per workgroup, split sequences).
 int fpk_compute_units() { return 8; }
