@@ -295,15 +295,23 @@ FP_DEVICE void score_weights(float s_intra, float lg, bool diagonal, bool revers
 // ---------------------------------------------------------------------------------------------
 // reverse workgroup: dk, dv, d_s0
 // PASS: 0 for waves 0..3 (dv), 1 for waves 4..7 (dk); the two copies meet at the same barriers.
+//
+// Per chunk, three stretches separated by workgroup barriers:
+//   1  what reads X (k or v): the score tile of this wave and the read-out of dS for its two output
+//      tiles, in one loop over the k-steps that shares the X operands; P goes to LDS
+//   2  Y^T += Z^T P^T and the outputs go to their staging tile; the state update; the k and v
+//      tiles of the next chunk replace the ones nobody reads any more; the new copy of dS
+//   3  the q and dO tiles of the next chunk
+// The outputs leave for global memory at the start of the next chunk's first stretch.
 template <int PASS>
 FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   using namespace fb;
   const Common k = make_common(p, stream);
-  uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // tiles: 0 q, 1 k, 2 v, 3 dO
+  uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // tiles: 0 q, 1 dO, 2 k, 3 v
   uint16_t* const Rt = TL + 4 * FB_TILE;                   // bf16(dS) as Rt[n = dv][a = dk]
   uint16_t* const OUT = Rt + FB_D * FB_LD;                 // staging: 0 dv, 1 dk
   uint16_t* const XP = OUT + 2 * FB_TILE;                  // score tiles [pass][tile][k-step][lane]
-  const uint16_t *Qs = TL, *Ks = TL + FB_TILE, *Vs = TL + 2 * FB_TILE, *Gs = TL + 3 * FB_TILE;
+  const uint16_t *Qs = TL, *Gs = TL + FB_TILE, *Ks = TL + 2 * FB_TILE, *Vs = TL + 3 * FB_TILE;
 
   constexpr int pass = PASS;
   const int rt = k.wave & 3, g = k.g, c = k.c, lane = k.lane;
@@ -315,11 +323,11 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   const float lg = k.lg;
 
   // score tile of this wave (rt < 3): (jb, ib) = (0,0), (1,0), (1,1); live entries have j >= i
+  const bool scores = rt < 3;
   const int s_jb = rt == 0 ? 0 : 1, s_ib = rt == 2 ? 1 : 0;
   float mw[16];
   score_weights(p.scale, lg, s_jb == s_ib, true, c, g, mw);
   const uint16_t* const s_wrow = Ws + at(32 * s_jb + score_row(c), 8 * g);
-  const uint16_t* const s_xrow = Xs + at(32 * s_ib + c, 8 * g);
 
   const TrLane tr_acc = tr_lane(lane, TR_ACC), tr_nat = tr_lane(lane, TR_NAT), tr_seq = tr_lane(lane, TR_SEQ);
   // state tiles of this wave: rows a = 32 at .., columns n = 32 (nt0 + {0, 1}) ..
@@ -334,12 +342,16 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   const float wread_full1 = p.scale * fprt::exp2_approx((float)(CH - 1 - 32 - c) * lg);
   const float gL_full = fprt::exp2_approx((float)CH * lg);
 
-  const void* const src[4] = {p.q, p.k, p.v, p.dO};
-  u32x4 pf[8];
-  load_tiles<4>(k, src, k.nch - 1, pf);
+  const void* const src_qg[2] = {p.q, p.dO};
+  const void* const src_kv[2] = {p.k, p.v};
+  u32x4 pf_qg[4], pf_kv[4];
+  load_tiles<2>(k, src_qg, k.nch - 1, pf_qg);
+  load_tiles<2>(k, src_kv, k.nch - 1, pf_kv);
   load_state(k, Rt, p.ds_out ? p.ds_out + (size_t)stream * FB_D * FB_D : nullptr, false);
-  stage_tiles<4>(k, TL, pf);
-  load_tiles<4>(k, src, k.nch - 2, pf);
+  stage_tiles<2>(k, TL, pf_qg);
+  stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
+  load_tiles<2>(k, src_qg, k.nch - 2, pf_qg);
+  load_tiles<2>(k, src_kv, k.nch - 2, pf_kv);
   fprt::block_sync();
   f32x16 racc[2];
 #pragma unroll
@@ -352,99 +364,52 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   for (int ci = k.nch - 1; ci >= 0; --ci) {
     const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
     fprt::prof_stamp(k.nch - 1 - ci, 0);
-    // ---- what the previous chunk left to do: its outputs leave, the copy of its dS is written.
-    // Nothing reads either buffer before the next barrier.
+    // ---- the previous chunk's outputs leave (nothing writes the staging tiles before the next barrier)
     if (ci < k.nch - 1) {
       drain_tile(k, OUT, p.dv, ci + 1);
       drain_tile(k, OUT + FB_TILE, p.dk, ci + 1);
-#pragma unroll
-      for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
     }
-    // ---- scores: the operands of a k-step are requested four k-steps ahead
-    if (rt < 3) {
-      ScoreFrags sf;
-      f32x16 sc = {0};
-#pragma unroll
-      for (int t = 0; t < 4; ++t) score_request(sf, s_wrow, s_xrow, t);
-      fprt::sched_fence();
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        sc = fprt::mfma_32x32x16_bf16(sf.w[t], sf.x[t], sc);
-        if (t < 4) score_request(sf, s_wrow, s_xrow, t + 4);
-        fprt::sched_fence();
-      }
-      score_finish(sc, mw, s_jb == s_ib, true, c, g, xp_pass + rt * FB_XP, lane);
-    }
-    fprt::prof_stamp(k.nch - 1 - ci, 1);
-    // ---- state update, dS[a][n] = gamma^L dS + sum_j gamma^(j+1) q[j][a] dO[j][n], operands two
-    // k-steps ahead
-    u32x4 ua[4], ub0[4], ub1[4];
-    auto request_u = [&](int t) {
-      ua[t] = frag_rows(Qs, tr_nat, t, 32 * at_);
-      ub0[t] = frag_rows(Gs, tr_nat, t, 32 * nt0);
-      ub1[t] = frag_rows(Gs, tr_nat, t, 32 * (nt0 + 1));
-    };
-    request_u(0);
-    request_u(1);
-    const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) racc[u][r] *= gL;
-    }
-    float wk[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) wk[e] = wk0[e];
-    fprt::sched_fence();
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const u32x4 wa = weigh(ua[t], wk);
-      racc[0] = fprt::mfma_32x32x16_bf16(wa, ub0[t], racc[0]);
-      racc[1] = fprt::mfma_32x32x16_bf16(wa, ub1[t], racc[1]);
-      if (t + 2 < 4) request_u(t + 2);
-      if (t < 3) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) wk[e] *= g16;
-      }
-      fprt::sched_fence();
-    }
-    fprt::prof_stamp(k.nch - 1 - ci, 2);
-    fprt::block_sync();
-    fprt::prof_stamp(k.nch - 1 - ci, 3);
-
-    // ---- outputs: Y^T[n][i] = wread(i) sum_a R^T[n][a] X[i][a] + sum_j Z^T[n][j] P^T[j][i]
-    // operands of the read-out in two batches, the second requested before the first is used;
-    // the operands of the intra-chunk part follow while the read-out's products run
-    f32x16 acc[2];
+    // ---- stretch 1: scores D[j][i] = W[j] . X[i] and read-out wread(i) sum_a R^T[n][a] X[i][a], the
+    // operands of a k-step requested a few k-steps ahead
+    f32x16 acc[2], sc = {0};
     acc[0] = f32x16{0};
     acc[1] = f32x16{0};
-    // the operands of k-step t + 4 are requested when those of k-step t are used
-    u32x4 ra[8], x0[8], x1[8];
-    auto request = [&](int t) {
-      // pass 0: R^T = dS^T[n][a] is a row of Rt; pass 1: R^T = dS[a][n] runs along the rows of Rt
-      ra[t] = pass == 0 ? frag_cols(rrow, t) : frag_rows(Rt, tr_seq, t, 32 * rt);
-      x0[t] = frag_cols(xrow0, t);
-      x1[t] = frag_cols(xrow1, t);
-    };
+    {
+      u32x4 wf[8], x0[8], x1[8], ra[8];
+      auto request = [&](int t) {
+        if (scores) wf[t] = frag_cols(s_wrow, t);
+        x0[t] = frag_cols(xrow0, t);
+        x1[t] = frag_cols(xrow1, t);
+        // pass 0: R^T = dS^T[n][a] is a row of Rt; pass 1: R^T = dS[a][n] runs along the rows of Rt
+        ra[t] = pass == 0 ? frag_cols(rrow, t) : frag_rows(Rt, tr_seq, t, 32 * rt);
+      };
+      constexpr int AHEAD = 3;   // k-steps of operands in flight
+      if (scores) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) request(t);
-    fprt::sched_fence();
+        for (int t = 0; t < AHEAD; ++t) request(t);
+        fprt::sched_fence();
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
-      acc[1] = fprt::mfma_32x32x16_bf16(ra[t], x1[t], acc[1]);
-      if (t + 4 < 8) request(t + 4);
-      fprt::sched_fence();
+        for (int t = 0; t < 8; ++t) {
+          sc = fprt::mfma_32x32x16_bf16(wf[t], s_ib ? x1[t] : x0[t], sc);
+          acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
+          acc[1] = fprt::mfma_32x32x16_bf16(ra[t], x1[t], acc[1]);
+          if (t + AHEAD < 8) request(t + AHEAD);
+          fprt::sched_fence();
+        }
+        score_finish(sc, mw, s_jb == s_ib, true, c, g, xp_pass + rt * FB_XP, lane);
+      } else {
+#pragma unroll
+        for (int t = 0; t < AHEAD; ++t) request(t);
+        fprt::sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
+          acc[1] = fprt::mfma_32x32x16_bf16(ra[t], x1[t], acc[1]);
+          if (t + AHEAD < 8) request(t + AHEAD);
+          fprt::sched_fence();
+        }
+      }
     }
-    u32x4 za[4], pq0[4], pq1[2];
-#pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-      za[tj] = frag_rows(Zs, tr_acc, tj, 32 * rt);
-      pq0[tj] = ld128(xp_pass + (tj >> 1) * FB_XP + 512 * (tj & 1) + lane * 8);
-      if (tj >= 2) pq1[tj - 2] = ld128(xp_pass + 2 * FB_XP + 512 * (tj & 1) + lane * 8);
-    }
-    fprt::sched_fence();
-    fprt::prof_stamp(k.nch - 1 - ci, 4);
     float wread0 = wread_full0, wread1 = wread_full1;
     if (L != CH) {   // the last chunk of the sequence, visited first
       const int e0 = L - 1 - c, e1 = L - 1 - 32 - c;
@@ -456,30 +421,80 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       acc[0][r] *= wread0;
       acc[1][r] *= wread1;
     }
-#pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-      acc[0] = fprt::mfma_32x32x16_bf16(za[tj], pq0[tj], acc[0]);
-      if (tj >= 2) acc[1] = fprt::mfma_32x32x16_bf16(za[tj], pq1[tj - 2], acc[1]);
-    }
-    put_output(out, c, 32 * rt, g, acc[0]);
-    put_output(out, 32 + c, 32 * rt, g, acc[1]);
-    fprt::prof_stamp(k.nch - 1 - ci, 5);
+    fprt::prof_stamp(k.nch - 1 - ci, 1);
     fprt::block_sync();
-    fprt::prof_stamp(k.nch - 1 - ci, 6);
+    fprt::prof_stamp(k.nch - 1 - ci, 2);
 
-    // ---- every read of this chunk's tiles is done: the next chunk's tiles take their place
-    stage_tiles<4>(k, TL, pf);
-    load_tiles<4>(k, src, ci - 2, pf);
-    fprt::prof_stamp(k.nch - 1 - ci, 7);
+    // ---- stretch 2: Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]
+    {
+      u32x4 za[4], pq0[4], pq1[2];
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        za[tj] = frag_rows(Zs, tr_acc, tj, 32 * rt);
+        pq0[tj] = ld128(xp_pass + (tj >> 1) * FB_XP + 512 * (tj & 1) + lane * 8);
+        if (tj >= 2) pq1[tj - 2] = ld128(xp_pass + 2 * FB_XP + 512 * (tj & 1) + lane * 8);
+      }
+      fprt::sched_fence();
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        acc[0] = fprt::mfma_32x32x16_bf16(za[tj], pq0[tj], acc[0]);
+        if (tj >= 2) acc[1] = fprt::mfma_32x32x16_bf16(za[tj], pq1[tj - 2], acc[1]);
+      }
+    }
+    // state update, dS[a][n] = gamma^L dS + sum_j gamma^(j+1) q[j][a] dO[j][n], operands two k-steps ahead
+    {
+      u32x4 ua[4], ub0[4], ub1[4];
+      auto request_u = [&](int t) {
+        ua[t] = frag_rows(Qs, tr_nat, t, 32 * at_);
+        ub0[t] = frag_rows(Gs, tr_nat, t, 32 * nt0);
+        ub1[t] = frag_rows(Gs, tr_nat, t, 32 * (nt0 + 1));
+      };
+      request_u(0);
+      request_u(1);
+      fprt::sched_fence();
+      put_output(out, c, 32 * rt, g, acc[0]);
+      put_output(out, 32 + c, 32 * rt, g, acc[1]);
+      const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) racc[u][r] *= gL;
+      }
+      float wk[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wk[e] = wk0[e];
+      fprt::sched_fence();
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const u32x4 wa = weigh(ua[t], wk);
+        racc[0] = fprt::mfma_32x32x16_bf16(wa, ub0[t], racc[0]);
+        racc[1] = fprt::mfma_32x32x16_bf16(wa, ub1[t], racc[1]);
+        if (t + 2 < 4) request_u(t + 2);
+        if (t < 3) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) wk[e] *= g16;
+        }
+        fprt::sched_fence();
+      }
+    }
+    fprt::prof_stamp(k.nch - 1 - ci, 3);
+    // nobody reads this chunk's k and v tiles or the old copy of dS any more
+    stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
+    load_tiles<2>(k, src_kv, ci - 2, pf_kv);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
+    fprt::prof_stamp(k.nch - 1 - ci, 4);
+    fprt::block_sync();
+    fprt::prof_stamp(k.nch - 1 - ci, 5);
+
+    // ---- stretch 3: every read of this chunk's q and dO tiles is done
+    stage_tiles<2>(k, TL, pf_qg);
+    load_tiles<2>(k, src_qg, ci - 2, pf_qg);
+    fprt::prof_stamp(k.nch - 1 - ci, 6);
     fprt::block_sync();
   }
   drain_tile(k, OUT, p.dv, 0);
   drain_tile(k, OUT + FB_TILE, p.dk, 0);
-  if (p.ds0) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
-    fprt::block_sync();
-  }
   if (p.ds0) store_state(k, Rt, p.ds0 + (size_t)stream * FB_D * FB_D, false);
 }
 
@@ -515,13 +530,17 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
 #else
   auto chunk_of = [&](int it) { return it; };
 #endif
-  const void* const src[3] = {p.dO, p.v, p.k};
-  u32x4 pf[6];
-  load_tiles<3>(k, src, chunk_of(0), pf);
+  const void* const src_x[1] = {p.dO};
+  const void* const src_wz[2] = {p.v, p.k};
+  u32x4 pf_x[2], pf_wz[4];
+  load_tiles<1>(k, src_x, chunk_of(0), pf_x);
+  load_tiles<2>(k, src_wz, chunk_of(0), pf_wz);
   // R[a][n] = S[n][a]: element (a, n) at n * 128 + a of s0
   load_state(k, Rt, p.s0 ? p.s0 + (size_t)stream * FB_D * FB_D : nullptr, true);
-  stage_tiles<3>(k, TL, pf);
-  load_tiles<3>(k, src, chunk_of(1), pf);
+  stage_tiles<1>(k, TL, pf_x);
+  stage_tiles<2>(k, TL + FB_TILE, pf_wz);
+  load_tiles<1>(k, src_x, chunk_of(1), pf_x);
+  load_tiles<2>(k, src_wz, chunk_of(1), pf_wz);
   fprt::block_sync();
   f32x16 racc[4];
   if constexpr (state_role) {
@@ -538,17 +557,16 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) wk_full[e] = p.scale * fprt::exp2_approx((float)(CH - 1 - (48 + nat_token(g, e))) * lg);
 
+  // Per chunk, three stretches separated by workgroup barriers, as in the reverse workgroup:
+  //   1  what reads X (dO): the read-out of R (output waves), the score tiles (state waves)
+  //   2  Y^T += Z^T P^T and the outputs (output waves); the state update and the new copy of R
+  //      (state waves); the next chunk's X tile
+  //   3  the next chunk's W and Z tiles
   for (int it = 0; it < k.nch; ++it) {
     const int ci = chunk_of(it);
     const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
-    // what the previous chunk left to do (nothing reads either buffer before the next barrier)
-    if (it > 0) {
-      drain_tile(k, OUT, p.dq, chunk_of(it - 1));
-      if constexpr (state_role) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) put_state(Rt, 32 * u + c, 32 * rt, g, racc[u]);
-      }
-    }
+    if (it > 0) drain_tile(k, OUT, p.dq, chunk_of(it - 1));   // nothing writes the staging tile before the next barrier
+    f32x16 acc[2];
     if constexpr (state_role) {
       if (rt < 3) {
         ScoreFrags sf;
@@ -564,47 +582,8 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
         }
         score_finish(sc, mw, s_jb == s_ib, false, c, g, XP + rt * FB_XP, lane);
       }
-      // R[a][n] = gamma^L R + sum_j s gamma^(L-1-j) W[j][a] Z[j][n]
-      const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) racc[u][r] *= gL;
-      }
-      // wkey(j) = s gamma^(L-1-j).  Full chunk: the last k-step's weights, times gamma^16 per
-      // earlier k-step.  Short chunk (the last one of a sequence): exponents clamped at 0 one by
-      // one (those rows are zero, the weight only has to stay finite).
-      float w[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) w[e] = wk_full[e];
-#pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const int t = 3 - tt;
-        if (L != CH) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const int x = L - 1 - (16 * t + nat_token(g, e));
-            w[e] = p.scale * fprt::exp2_approx((float)(x > 0 ? x : 0) * lg);
-          }
-        }
-        u32x4 ub[4];
-        const u32x4 ua = frag_rows(Ws, tr_nat, t, 32 * rt);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) ub[u] = frag_rows(Zs, tr_nat, t, 32 * u);
-        const u32x4 wa = weigh(ua, w);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) racc[u] = fprt::mfma_32x32x16_bf16(wa, ub[u], racc[u]);
-        if (tt < 3) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) w[e] *= g16;
-        }
-      }
-    }
-    fprt::block_sync();
-
-    if constexpr (!state_role) {
-      // Y^T[n][i] = gamma^(i+1) sum_a R^T[n][a] X[i][a] + sum_j Z^T[n][j] P^T[j][i]
-      f32x16 acc[2];
+    } else {
+      // Y^T[n][i] = gamma^(i+1) sum_a R^T[n][a] X[i][a]
       acc[0] = f32x16{0};
       acc[1] = f32x16{0};
       u32x4 ra[8], x0[8], x1[8];
@@ -623,7 +602,17 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
         if (t + 4 < 8) request(t + 4);
         fprt::sched_fence();
       }
-      // tokens j < 32 reach both halves (tiles (0,0), (0,1)), the others only the second
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[0][r] *= wread0;
+        acc[1][r] *= wread1;
+      }
+    }
+    fprt::block_sync();
+
+    if constexpr (!state_role) {
+      // Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]; tokens j < 32 reach both halves (tiles (0,0), (0,1)),
+      // the others only the second
       u32x4 za[4], pq1[4], pq0[2];
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) {
@@ -633,22 +622,65 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
       }
       fprt::sched_fence();
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc[0][r] *= wread0;
-        acc[1][r] *= wread1;
-      }
-#pragma unroll
       for (int tj = 0; tj < 4; ++tj) {
         acc[1] = fprt::mfma_32x32x16_bf16(za[tj], pq1[tj], acc[1]);
         if (tj < 2) acc[0] = fprt::mfma_32x32x16_bf16(za[tj], pq0[tj], acc[0]);
       }
       put_output(OUT, c, 32 * rt, g, acc[0]);
       put_output(OUT, 32 + c, 32 * rt, g, acc[1]);
+    } else {
+      // R[a][n] = gamma^L R + sum_j s gamma^(L-1-j) W[j][a] Z[j][n]
+      const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) racc[u][r] *= gL;
+      }
+      // wkey(j) = s gamma^(L-1-j).  Full chunk: the last k-step's weights, times gamma^16 per
+      // earlier k-step.  Short chunk (the last one of a sequence): exponents clamped at 0 one by
+      // one (those rows are zero, the weight only has to stay finite).
+      float w[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w[e] = wk_full[e];
+      u32x4 ua[4], ub[4][4];
+      auto request_u = [&](int t) {
+        ua[t] = frag_rows(Ws, tr_nat, t, 32 * rt);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) ub[t][u] = frag_rows(Zs, tr_nat, t, 32 * u);
+      };
+      request_u(3);
+      request_u(2);
+      fprt::sched_fence();
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        const int t = 3 - tt;
+        if (L != CH) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int x = L - 1 - (16 * t + nat_token(g, e));
+            w[e] = p.scale * fprt::exp2_approx((float)(x > 0 ? x : 0) * lg);
+          }
+        }
+        const u32x4 wa = weigh(ua[t], w);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) racc[u] = fprt::mfma_32x32x16_bf16(wa, ub[t][u], racc[u]);
+        if (t >= 2) request_u(t - 2);
+        if (tt < 3) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e] *= g16;
+        }
+        fprt::sched_fence();
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) put_state(Rt, 32 * u + c, 32 * rt, g, racc[u]);
     }
+    // nobody reads this chunk's X tile any more
+    stage_tiles<1>(k, TL, pf_x);
+    load_tiles<1>(k, src_x, chunk_of(it + 2), pf_x);
     fprt::block_sync();
 
-    stage_tiles<3>(k, TL, pf);
-    load_tiles<3>(k, src, chunk_of(it + 2), pf);
+    stage_tiles<2>(k, TL + FB_TILE, pf_wz);
+    load_tiles<2>(k, src_wz, chunk_of(it + 2), pf_wz);
     fprt::block_sync();
   }
   drain_tile(k, OUT, p.dq, chunk_of(k.nch - 1));
