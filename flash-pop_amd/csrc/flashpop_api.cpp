@@ -179,6 +179,7 @@ int forward(const Shape& s, const void* q, const void* k, const void* v, const v
 // environment overrides the choice (for A/B measurements).
 bool use_fused_backward(const Shape& s, const void* d_blocks) {
   if (s.dk != fpk::FB_D || s.dv != fpk::FB_D || d_blocks) return false;
+  if (s.T < 8 * fpk::CH) return false;   // short sequences: the walk over many of them per workgroup serves better
   if (const char* e = std::getenv("FLASHPOP_BWD")) {
     if (std::strcmp(e, "passes") == 0) return false;
     if (std::strcmp(e, "fused") == 0) return true;
@@ -186,10 +187,23 @@ bool use_fused_backward(const Shape& s, const void* d_blocks) {
   return 4LL * s.B * s.H >= fpk_compute_units();
 }
 
+// Tokens between the states that fp_retention_fwd_ckpt leaves for the backward (0: none wanted).
+// Eight chunks: the checkpoints cost 1/16 of the forward's traffic, and the segment that the two
+// workgroups of a stream share stays within reach of the caches.
+int checkpoint_interval(const Shape& s) {
+  int every = 8 * fpk::CH;
+  if (const char* e = std::getenv("FLASHPOP_CKPT")) every = std::atoi(e) / fpk::CH * fpk::CH;
+  if (every <= 0 || !use_fused_backward(s, nullptr) || s.T <= every) return 0;
+  return every;
+}
+
 int backward_fused(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
-                   const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, void* stream) {
+                   const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, void* stream,
+                   const void* ckpt = nullptr, int ckpt_every = 0) {
   fpk::FusedBwdArgs a;
   std::memset(&a, 0, sizeof a);
+  a.ckpt = in(ckpt);
+  a.ckpt_every = ckpt ? ckpt_every : 0;
   a.q = in(q); a.k = in(k); a.v = in(v); a.dO = in(d_o);
   a.dq = out(dq); a.dk = out(dk_); a.dv = out(dv_);
   a.s0 = in(s0); a.ds_out = in(d_s_out); a.ds0 = out(d_s0);
@@ -464,6 +478,40 @@ int fp_retention_bwd(const void* q, const void* k, const void* v, const void* s0
   return backward(s, q, k, v, s0, head_decays, d_o, d_s_out, nullptr, 0, dq, dk_, dv_, d_s0, stream);
 }
 
+size_t fp_retention_checkpoint_bytes(int B, int T, int H, int dk, int dv, int* every) {
+  const Shape s{B, T, H, dk, dv};
+  if (every) *every = 0;
+  if (B < 1 || T < 1 || H < 1 || H > fpk::MAX_HEADS || !dim_ok(dk) || !dim_ok(dv)) return 0;
+  const int n = checkpoint_interval(s);
+  if (n <= 0) return 0;
+  if (every) *every = n;
+  return sizeof(uint16_t) * (size_t)B * (T / n) * H * dk * dv;
+}
+
+int fp_retention_fwd_ckpt(const void* q, const void* k, const void* v, const void* s0, const double* head_decays, void* o,
+                          void* s_out, void* checkpoints, int every, int B, int T, int H, int dk, int dv, void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
+  if (!checkpoints || every <= 0) return forward(s, q, k, v, s0, head_decays, o, s_out, nullptr, 0, stream);
+  if (every % fpk::CH != 0) return fail(FP_ERR_BAD_SHAPE, "the checkpoint interval must be a multiple of %d tokens (got %d)", fpk::CH, every);
+  return forward(s, q, k, v, s0, head_decays, o, s_out, T / every > 0 ? checkpoints : nullptr, every, stream);
+}
+
+int fp_retention_bwd_ckpt(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                          const void* d_o, const void* d_s_out, const void* checkpoints, int every, void* dq, void* dk_,
+                          void* dv_, void* d_s0, int B, int T, int H, int dk, int dv, void* stream) {
+  const Shape s{B, T, H, dk, dv};
+  if (int rc = check_shape(s, head_decays)) return rc;
+  if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
+    return fail(FP_ERR_NULL_POINTER, "q, k, v, d_o, dq, dk and dv must not be NULL");
+  if (checkpoints && (every <= 0 || every % fpk::CH != 0))
+    return fail(FP_ERR_BAD_SHAPE, "the checkpoint interval must be a positive multiple of %d tokens (got %d)", fpk::CH, every);
+  if (checkpoints && T / every > 0 && use_fused_backward(s, nullptr))
+    return backward_fused(s, q, k, v, s0, head_decays, d_o, d_s_out, dq, dk_, dv_, d_s0, stream, checkpoints, every);
+  return backward(s, q, k, v, s0, head_decays, d_o, d_s_out, nullptr, 0, dq, dk_, dv_, d_s0, stream);
+}
+
 size_t fp_retention_workspace_bytes(int B, int T, int H, int dk, int dv) {
   const Shape s{B, T, H, dk, dv};
   if (B < 1 || T < 1 || H < 1 || H > fpk::MAX_HEADS || !dim_ok(dk) || !dim_ok(dv)) return 0;
@@ -655,6 +703,6 @@ int fp_probe_stream_pattern(const void* x, const void* w, const void* z, void* y
 
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1005; }
+int fp_version(void) { return 1006; }
 
 }  // extern "C"

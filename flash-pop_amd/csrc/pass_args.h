@@ -114,6 +114,13 @@ struct FusedBwdArgs {
   const uint16_t* s0;                      // [B,H,128,128], nullable (zeros)
   const uint16_t* ds_out;                  // gradient of the final state, nullable (zeros)
   uint16_t* ds0;                           // gradient of s0, nullable (not wanted)
+  // States that the forward pass left behind every `ckpt_every` tokens (a multiple of 64):
+  // ckpt[b][m][h] is the state after token (m + 1) * ckpt_every - 1, m < T / ckpt_every.  With them
+  // the dq workgroup takes the segments between them from the last to the first (forward inside a
+  // segment), next to the reverse workgroup of its stream, so that what one of the two fetches
+  // the other finds in the caches.  Null: one forward walk from s0.
+  const uint16_t* ckpt;
+  int ckpt_every;
   int B, T, H;
   float scale;                             // dk^-1/2
   float log2g[MAX_HEADS];

@@ -525,18 +525,32 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
   const uint16_t* const s_xrow = Xs + at(32 * s_ib + c, 8 * g);
   const TrLane tr_acc = tr_lane(lane, TR_ACC), tr_nat = tr_lane(lane, TR_NAT);
 
-#ifdef FB_SEGREV
-  auto chunk_of = [&](int it) { const int seg = k.nch / FB_SEGREV - 1 - it / FB_SEGREV; return it < 0 || it >= k.nch ? -1 : seg * FB_SEGREV + it % FB_SEGREV; };
-#else
-  auto chunk_of = [&](int it) { return it; };
-#endif
+  // The walk: without checkpoints the chunks in order; with them the segments from the last to the
+  // first, the chunks of a segment in order.  seg_chunks = chunks per segment.
+  const int seg_chunks = p.ckpt ? p.ckpt_every / CH : k.nch;
+  const int nseg = (k.nch + seg_chunks - 1) / seg_chunks;
+  auto chunk_of = [&](int it) {   // chunk visited in iteration `it`, -1 beyond the walk
+    if (it < 0 || it >= k.nch) return -1;
+    if (nseg == 1) return it;
+    // the last segment may be shorter than the others
+    const int tail = k.nch - (nseg - 1) * seg_chunks;
+    if (it < tail) return (nseg - 1) * seg_chunks + it;
+    const int j = it - tail;
+    return (nseg - 2 - j / seg_chunks) * seg_chunks + j % seg_chunks;
+  };
+  // state matrix that a segment starts from: s0 for the first, else the checkpoint before it
+  auto segment_state = [&](int seg) -> const uint16_t* {
+    if (seg == 0) return p.s0 ? p.s0 + (size_t)stream * FB_D * FB_D : nullptr;
+    const size_t nck = (size_t)(k.T / p.ckpt_every);
+    return p.ckpt + (((size_t)k.b * nck + (seg - 1)) * p.H + k.h) * FB_D * FB_D;
+  };
   const void* const src_x[1] = {p.dO};
   const void* const src_wz[2] = {p.v, p.k};
   u32x4 pf_x[2], pf_wz[4];
   load_tiles<1>(k, src_x, chunk_of(0), pf_x);
   load_tiles<2>(k, src_wz, chunk_of(0), pf_wz);
-  // R[a][n] = S[n][a]: element (a, n) at n * 128 + a of s0
-  load_state(k, Rt, p.s0 ? p.s0 + (size_t)stream * FB_D * FB_D : nullptr, true);
+  // R[a][n] = S[n][a]: element (a, n) at n * 128 + a of a state matrix
+  load_state(k, Rt, segment_state(nseg - 1), true);
   stage_tiles<1>(k, TL, pf_x);
   stage_tiles<2>(k, TL + FB_TILE, pf_wz);
   load_tiles<1>(k, src_x, chunk_of(1), pf_x);
@@ -563,7 +577,8 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
   //      (state waves); the next chunk's X tile
   //   3  the next chunk's W and Z tiles
   for (int it = 0; it < k.nch; ++it) {
-    const int ci = chunk_of(it);
+    const int ci = chunk_of(it), next = chunk_of(it + 1);
+    const bool fresh = next >= 0 && next != ci + 1;   // the next chunk starts another segment
     const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
     if (it > 0) drain_tile(k, OUT, p.dq, chunk_of(it - 1));   // nothing writes the staging tile before the next barrier
     f32x16 acc[2];
@@ -671,16 +686,25 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
         }
         fprt::sched_fence();
       }
+      if (!fresh) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) put_state(Rt, 32 * u + c, 32 * rt, g, racc[u]);
+        for (int u = 0; u < 4; ++u) put_state(Rt, 32 * u + c, 32 * rt, g, racc[u]);
+      }
     }
-    // nobody reads this chunk's X tile any more
+    // nobody reads this chunk's X tile or the old copy of R any more
     stage_tiles<1>(k, TL, pf_x);
     load_tiles<1>(k, src_x, chunk_of(it + 2), pf_x);
+    if (fresh) load_state(k, Rt, segment_state(next / seg_chunks), true);   // the next segment's starting state
     fprt::block_sync();
 
     stage_tiles<2>(k, TL + FB_TILE, pf_wz);
     load_tiles<2>(k, src_wz, chunk_of(it + 2), pf_wz);
+    if constexpr (state_role) {
+      if (fresh) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) racc[u] = get_state(Rt, 32 * u + c, 32 * rt, g);
+      }
+    }
     fprt::block_sync();
   }
   drain_tile(k, OUT, p.dq, chunk_of(k.nch - 1));

@@ -17,6 +17,9 @@ _L, _F = c_longlong, c_double
 SIGNATURES = {
     "fp_retention_fwd": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P],
     "fp_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "fp_retention_checkpoint_bytes": [_I, _I, _I, _I, _I, POINTER(c_int)],
+    "fp_retention_fwd_ckpt": [_P, _P, _P, _P, _D, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "fp_retention_bwd_ckpt": [_P, _P, _P, _P, _D, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
     "fp_retention_workspace_bytes": [_I, _I, _I, _I, _I],
     "fp_retention_fwd_split": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
     "fp_retention_fwd_split_static": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P],
@@ -43,7 +46,8 @@ def bind(path: str) -> ctypes.CDLL:
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
         fn.argtypes = argtypes
-        fn.restype = {"fp_last_error": c_char_p, "fp_retention_workspace_bytes": c_size_t}.get(name, c_int)
+        fn.restype = {"fp_last_error": c_char_p, "fp_retention_workspace_bytes": c_size_t,
+                      "fp_retention_checkpoint_bytes": c_size_t}.get(name, c_int)
     return lib
 
 

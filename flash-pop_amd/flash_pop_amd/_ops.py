@@ -1,6 +1,8 @@
 """Tensor-level plumbing shared by the two autograd Functions: checks, allocation, raw calls."""
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -54,22 +56,34 @@ def _workspace(lib, shape, device):
     return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
 
 
-def retention_fwd(q, k, v, s, decays, shape):
+def retention_fwd(q, k, v, s, decays, shape, for_backward=False):
+    """-> (o, s_out, checkpoints or None, checkpoint interval).  With `for_backward` the forward
+    also leaves the states that make the backward cheaper, where the library says they pay."""
     refuse_capture("retention_fwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
     o = torch.empty((B, T, H, dv), dtype=q.dtype, device=q.device)
     s_out = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device)
+    ckpt, every = None, 0
     with torch.cuda.device(q.device):
         ws = _workspace(lib, shape, q.device)
-        if ws is None:
+        if ws is None and for_backward:
+            n = ctypes.c_int(0)
+            nbytes = lib.fp_retention_checkpoint_bytes(B, T, H, dk, dv, ctypes.byref(n))
+            if nbytes:
+                every = n.value
+                ckpt = torch.empty((B, T // every, H, dk, dv), dtype=q.dtype, device=q.device)
+        if ckpt is not None:
+            rc = lib.fp_retention_fwd_ckpt(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
+                                           _ptr(s_out), _ptr(ckpt), every, B, T, H, dk, dv, _stream())
+        elif ws is None:
             rc = lib.fp_retention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
                                       _ptr(s_out), B, T, H, dk, dv, _stream())
         else:
             rc = lib.fp_retention_fwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
                                             _ptr(s_out), B, T, H, dk, dv, _ptr(ws), ws.numel(), _stream())
     _lib.check(lib, rc)
-    return o, s_out
+    return o, s_out, ckpt, every
 
 
 def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
@@ -85,8 +99,9 @@ def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
     return o, states
 
 
-def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0):
-    """Gradients for both ops; block_size is None for the plain op."""
+def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0, ckpt=None, every=0):
+    """Gradients for both ops; block_size is None for the plain op.  ckpt, every: what retention_fwd
+    left for this call."""
     refuse_capture("retention_bwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
@@ -97,7 +112,11 @@ def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size,
     d_s0 = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device) if want_ds0 else None
     with torch.cuda.device(q.device):
         ws = _workspace(lib, shape, q.device) if block_size is None else None
-        if ws is not None:
+        if ckpt is not None and block_size is None:
+            rc = lib.fp_retention_bwd_ckpt(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
+                                           _ptr(d_s_out), _ptr(ckpt), every, _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0),
+                                           B, T, H, dk, dv, _stream())
+        elif ws is not None:
             rc = lib.fp_retention_bwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                             _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
                                             _ptr(ws), ws.numel(), _stream())

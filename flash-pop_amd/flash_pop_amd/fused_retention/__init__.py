@@ -16,17 +16,24 @@ class FusedChunkRetention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, s, head_decays):
         q, k, v, s, shape = _ops.prepare(q, k, v, s, head_decays)
-        o, s_out = _ops.retention_fwd(q, k, v, s, head_decays, shape)
-        ctx.save_for_backward(q, k, v, s)
+        # what the reference saves for its backward (fused_retention/__init__.py:30) plus, where it
+        # pays, the states the forward passes through every few chunks
+        o, s_out, ckpt, every = _ops.retention_fwd(q, k, v, s, head_decays, shape, for_backward=any(ctx.needs_input_grad[:4]))
+        ctx.save_for_backward(q, k, v, s, ckpt)
+        ctx.set_materialize_grads(False)   # an output nobody differentiates arrives as None, not as a tensor of zeros
+        ctx.every = every
         ctx.head_decays = tuple(head_decays)
         ctx.shape = shape
         return o, s_out
 
     @staticmethod
     def backward(ctx, d_o, d_s_out):
-        q, k, v, s = ctx.saved_tensors
+        q, k, v, s, ckpt = ctx.saved_tensors
+        if d_o is None:
+            d_o = torch.zeros((*q.shape[:3], v.shape[3]), dtype=q.dtype, device=q.device)
         want_ds0 = s is not None and ctx.needs_input_grad[3]
-        dq, dk, dv, d_s0 = _ops.retention_bwd(q, k, v, s, ctx.head_decays, ctx.shape, d_o, d_s_out, None, None, want_ds0)
+        dq, dk, dv, d_s0 = _ops.retention_bwd(q, k, v, s, ctx.head_decays, ctx.shape, d_o, d_s_out, None, None, want_ds0,
+                                              ckpt, ctx.every)
         return dq, dk, dv, d_s0, None
 
 

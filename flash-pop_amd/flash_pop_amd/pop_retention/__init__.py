@@ -30,6 +30,7 @@ class FlashPOPRetention(torch.autograd.Function):
         q, k, v, s, shape = _ops.prepare(q, k, v, s, head_decays)
         o, states = _ops.pop_retention_fwd(q, k, v, s, head_decays, block_size, shape)
         ctx.save_for_backward(q, k, v, s)
+        ctx.set_materialize_grads(False)   # an output nobody differentiates arrives as None, not as a tensor of zeros
         ctx.head_decays = tuple(head_decays)
         ctx.shape = shape
         ctx.block_size = block_size
@@ -38,6 +39,8 @@ class FlashPOPRetention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_o, d_block_states):
         q, k, v, s = ctx.saved_tensors
+        if d_o is None:
+            d_o = torch.zeros((*q.shape[:3], v.shape[3]), dtype=q.dtype, device=q.device)
         want_ds0 = s is not None and ctx.needs_input_grad[3]
         dq, dk, dv, d_s0 = _ops.retention_bwd(q, k, v, s, ctx.head_decays, ctx.shape, d_o, None, d_block_states,
                                               ctx.block_size, want_ds0)
@@ -57,6 +60,7 @@ class FlashPOPRetentionWithSuffixes(torch.autograd.Function):
         sfx = _ops.prepare_suffixes(q_sfx, k_sfx, v_sfx, shape, block_size)
         o, o_sfx, last_state = _ops.pop_fused_fwd(q, k, v, s, sfx, head_decays, block_size, shape)
         ctx.save_for_backward(q, k, v, s, *sfx)
+        ctx.set_materialize_grads(False)   # an output nobody differentiates arrives as None, not as a tensor of zeros
         ctx.head_decays = tuple(head_decays)
         ctx.shape = shape
         ctx.block_size = block_size
@@ -65,6 +69,10 @@ class FlashPOPRetentionWithSuffixes(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_o, d_o_sfx, d_last_state):
         q, k, v, s, *sfx = ctx.saved_tensors
+        if d_o is None:
+            d_o = torch.zeros((*q.shape[:3], v.shape[3]), dtype=q.dtype, device=q.device)
+        if d_o_sfx is None:
+            d_o_sfx = torch.zeros((*sfx[0].shape[:3], v.shape[3]), dtype=q.dtype, device=q.device)
         want_ds0 = s is not None and ctx.needs_input_grad[3]
         (dq, dk, dv, dq_s, dk_s, dv_s), d_s0 = _ops.pop_fused_bwd(q, k, v, s, sfx, ctx.head_decays, ctx.block_size,
                                                                    ctx.shape, d_o, d_o_sfx, d_last_state, want_ds0)

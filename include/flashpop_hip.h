@@ -52,6 +52,28 @@ int fp_retention_bwd(const void* q, const void* k, const void* v, const void* s0
                      const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B, int T,
                      int H, int dk, int dv, void* stream);
 
+/* Forward and backward with checkpoints.  The backward needs the state at the start of every
+ * chunk for dq and gets it by re-running the recurrence forward (as the reference's
+ * fused_retention_bwd_dq does, fused_chunk_bwd.py:432-444), which walks against the reverse
+ * recurrence of dk and dv and reads k, v and d_o a second time from HBM.  When the forward leaves
+ * its state every `every` tokens, the backward takes the segments between those states from the
+ * last to the first, beside the reverse walk, and the second read comes from the caches.  What
+ * FusedChunkRetention saves for its backward (fused_retention/__init__.py:30) grows by these states.
+ *   fp_retention_checkpoint_bytes  bytes of the checkpoint buffer that pays for this shape on the
+ *                                  current device and, in *every, the interval in tokens; 0 when the
+ *                                  shape is served as well without (then pass NULL below)
+ *   checkpoints  [B, T / every, H, dk, dv] bf16: the state after tokens every - 1, 2 every - 1, ...;
+ *                written by _fwd_ckpt, read by _bwd_ckpt.  NULL: same as fp_retention_fwd / _bwd.
+ *   every        a multiple of 64
+ * Results are those of fp_retention_fwd / fp_retention_bwd up to the rounding of the checkpoints
+ * to bf16 (dq only). */
+size_t fp_retention_checkpoint_bytes(int B, int T, int H, int dk, int dv, int* every);
+int fp_retention_fwd_ckpt(const void* q, const void* k, const void* v, const void* s0, const double* head_decays, void* o,
+                          void* s_out, void* checkpoints, int every, int B, int T, int H, int dk, int dv, void* stream);
+int fp_retention_bwd_ckpt(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
+                          const void* d_o, const void* d_s_out, const void* checkpoints, int every, void* dq, void* dk_,
+                          void* dv_, void* d_s0, int B, int T, int H, int dk, int dv, void* stream);
+
 /* Long sequences with few (batch, head) streams: one workgroup walks one stream, so B * H *
  * min(dk, dv) / 64 workgroups is all a call has, and a 256-CU device idles when that is small.
  * The _split variants cut every sequence into segments that run as separate sequences (a

@@ -332,3 +332,18 @@ def raw_stream_probe(lib, x, w, z, stream=None):
     y = torch.full_like(z, float("nan"))
     _check(lib, lib.fp_probe_stream_pattern(_p(x), _p(w), _p(z), _p(y), B, T, H, dA, z.shape[3], stream))
     return y
+
+
+def raw_ckpt_fwd_bwd(lib, q, k, v, s, decays, d_o, d_s, every, stream=None):
+    """fp_retention_fwd_ckpt followed by fp_retention_bwd_ckpt with checkpoints every `every` tokens.
+    Returns (o, S, dq, dk, dv, ds0)."""
+    B, T, H, dk = q.shape
+    dv = v.shape[3]
+    nan = lambda *shape: torch.full(shape, float("nan"), dtype=BF16, device=q.device)
+    o, S, ck = nan(B, T, H, dv), nan(B, H, dk, dv), nan(B, T // every, H, dk, dv)
+    _check(lib, lib.fp_retention_fwd_ckpt(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o), _p(S), _p(ck) if ck.numel() else None,
+                                          every, B, T, H, dk, dv, stream))
+    dq, dk_, dv_, ds0 = nan(*q.shape), nan(*k.shape), nan(*v.shape), nan(B, H, dk, dv)
+    _check(lib, lib.fp_retention_bwd_ckpt(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(d_o), _p(d_s), _p(ck) if ck.numel() else None,
+                                          every, _p(dq), _p(dk_), _p(dv_), _p(ds0), B, T, H, dk, dv, stream))
+    return o, S, dq, dk_, dv_, ds0

@@ -31,7 +31,7 @@ def test_header_and_binding_agree(lib):
     assert names == sorted(_lib.SIGNATURES), (names, sorted(_lib.SIGNATURES))
     for n in names:
         assert hasattr(lib, n), f"{n} not exported"
-    assert lib.fp_version() == 1005
+    assert lib.fp_version() == 1006
 
 
 def test_argument_checks_return_codes(lib):

@@ -107,6 +107,51 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
 
 
+@pytest.mark.parametrize("B,T,H,state_std,every", [
+    (1, 700, 2, 0.5, 128),      # ragged tail beyond the last checkpoint, initial state
+    (1, 512, 1, None, 256),     # the sequence ends on a checkpoint, no initial state
+    (2, 520, 1, 0.3, 64),       # a checkpoint after every chunk, two sequences
+    (1, 600, 1, 0.2, 1024),     # interval longer than the sequence: no checkpoint at all
+    (1, 576, 2, 0.4, 0),        # no checkpoint buffer: the fused backward walks forward from s0
+])
+def test_fused_backward_with_checkpoints(emu_lib, monkeypatch, B, T, H, state_std, every):
+    """dk = dv = 128 and at least eight chunks: the backward that carries dS once, beside the
+    workgroup that re-runs the state from the checkpoints the forward left (segments taken from
+    the last to the first)."""
+    monkeypatch.setenv("FLASHPOP_BWD", "fused")
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, 128, 128, seed=T, state_std=state_std)
+    d_o, d_s = hp.make_cotangents([(B, T, H, 128), (B, H, 128, 128)], seed=T + 1)
+    if every:
+        o, S, dq, dk_, dv_, ds0 = hp.raw_ckpt_fwd_bwd(emu_lib, q, k, v, s, decays, d_o, d_s, every)
+    else:
+        o, S = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+        dq, dk_, dv_, ds0 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
+    o_ref, S_ref, (gq, gk, gv, gs) = hp.oracle_plain(q, k, v, s, decays, d_o, d_s)
+    _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
+    # the checkpoints only serve dq: everything else is bit for bit what the entry points without them give
+    o2, S2 = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+    g2 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
+    assert torch.equal(o, o2) and torch.equal(S, S2)
+    assert torch.equal(dk_, g2[1]) and torch.equal(dv_, g2[2])
+    assert (ds0 is None and g2[3] is None) or torch.equal(ds0, g2[3])
+
+
+def test_checkpoint_size_query(emu_lib, monkeypatch):
+    """fp_retention_checkpoint_bytes: 0 where the fused backward would not run or the sequence is
+    no longer than one interval, else B * (T / every) state matrices."""
+    import ctypes
+    every = ctypes.c_int(-1)
+    monkeypatch.setenv("FLASHPOP_BWD", "fused")
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 2 * 2 * (4096 // 512) * 4 * 128 * 128
+    assert every.value == 512
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 512, 4, 128, 128, ctypes.byref(every)) == 0 and every.value == 0
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 64, 128, ctypes.byref(every)) == 0
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, None) > 0
+    monkeypatch.setenv("FLASHPOP_BWD", "passes")
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 0
+
+
 @pytest.mark.parametrize("B,H,dk,dv", [(2, 3, 64, 128), (1, 2, 128, 64), (1, 1, 256, 256)])
 def test_decode_step(emu_lib, B, H, dk, dv):
     """Three chained steps (no state, fresh buffer, in place) against the oracle's recurrent step."""

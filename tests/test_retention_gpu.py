@@ -94,6 +94,31 @@ def test_config3_long_context_carried_state():
         for n in ("o", "S", "dq", "dk", "dv", "ds0")))
 
 
+def test_checkpointed_backward_against_oracle_and_plain_entry_points(hip_lib):
+    """fp_retention_fwd_ckpt / fp_retention_bwd_ckpt on a shape that takes the fused backward
+    (dk = dv = 128, enough streams): all results against the oracle; o, S, dk, dv and ds0 bit for bit
+    those of the entry points without checkpoints (the checkpoints only serve dq)."""
+    import ctypes
+    B, T, H = 4, 1600, 16
+    decays = oracle.head_decays(H)
+    q, k, v, s = (t.to(DEV) for t in hp.make_inputs(B, T, H, 128, 128, seed=11, state_std=0.3))
+    d_o, d_s = (t.to(DEV) for t in hp.make_cotangents([(B, T, H, 128), (B, H, 128, 128)], seed=12))
+    n = ctypes.c_int(0)
+    nbytes = hip_lib.fp_retention_checkpoint_bytes(B, T, H, 128, 128, ctypes.byref(n))
+    assert n.value > 0 and nbytes == 2 * B * (T // n.value) * H * 128 * 128, "this shape is meant to take the checkpointed path"
+    plain = hp.raw_fwd(hip_lib, q, k, v, s, decays) + hp.raw_bwd(hip_lib, q, k, v, s, decays, d_o, d_s)
+    for every in (n.value, 64, 448):
+        _say(f"[checkpoints] B{B} T{T} H{H} every {every}")
+        got = hp.raw_ckpt_fwd_bwd(hip_lib, q, k, v, s, decays, d_o, d_s, every)
+        torch.cuda.synchronize()
+        o_ref, S_ref, grads = hp.oracle_plain(q, k, v, s, decays, d_o, d_s, device=DEV)
+        for name, g, ref in zip(("o", "S", "dq", "dk", "dv", "ds0"), got, (o_ref, S_ref, *grads)):
+            hp.assert_close(g, ref, f"{name} (every {every})", head_dim=1 if name in ("S", "ds0") else 2)
+        for i, name in enumerate(("o", "S", "dq", "dk", "dv", "ds0")):
+            if name != "dq":
+                assert torch.equal(got[i], plain[i]), name
+
+
 def test_split_sequence_equals_one_run_at_full_size():
     """Running [0, T1) then [T1, T) with the carried state must reproduce the single run up to the
     bf16 rounding of the hand-over state (size-independent property, config-2 shape)."""
@@ -166,6 +191,29 @@ def test_state_none_equals_zero_state_and_grad_flags():
     o3, _ = fused_chunk_retention(ql, k, v, z, decays)
     o3.float().sum().backward()
     assert ql.grad is not None and ql.grad.shape == q.shape
+
+
+def test_gradient_through_the_final_state_only():
+    """Only S is differentiated: the op receives no d_o (it is not materialised as zeros by autograd)
+    and must behave as if it were zero; likewise for the POP op's block states."""
+    from flash_pop_amd import fused_chunk_retention, flash_pop_retention
+    B, T, H, d = 2, 150, 2, 128
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, d, d, seed=21, state_std=0.3)
+    d_s, = hp.make_cotangents([(B, H, d, d)], seed=22)
+    leaves = [t.to(DEV).requires_grad_() for t in (q, k, v, s)]
+    _, S = fused_chunk_retention(*leaves, decays)
+    S.backward(d_s.to(DEV))
+    _, _, grads = hp.oracle_plain(q, k, v, s, decays, torch.zeros(B, T, H, d), d_s)
+    for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), leaves, grads):
+        hp.assert_close(leaf.grad, ref, name, head_dim=1 if name == "ds0" else 2)
+    leaves = [t.to(DEV).requires_grad_() for t in (q, k, v, s)]
+    _, states = flash_pop_retention(*leaves, decays, 64)
+    d_states, = hp.make_cotangents([tuple(states.shape)], seed=23)
+    states.backward(d_states.to(DEV))
+    _, _, grads = hp.oracle_pop(q, k, v, s, decays, 64, torch.zeros(B, T, H, d), d_states)
+    for name, leaf, ref in zip(("dq", "dk", "dv", "ds0"), leaves, grads):
+        hp.assert_close(leaf.grad, ref, "pop " + name, head_dim=1 if name == "ds0" else 2)
 
 
 def test_recurrent_decode_matches_chunkwise():
