@@ -3,10 +3,11 @@
 A step is one forward + backward of fused_chunk_retention over one synthetic batch of
 benchmark configuration 2 (bf16, B=8 H=16 T=4096 dk=dv=128, zero initial state, dO ~ N(0,1)), inputs
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic FLOP count
-(dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the pass kernel measured
-with events on the launch stream, and the CPU oracle timed on the host cores beside it.
+(dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the backward kernel (the
+dominant launch of a step) measured with events on the launch stream, and the CPU oracle timed on
+the host cores beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-pop] [--no-long] [--no-layer] [--no-model]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--spin-up S] [--no-cpu] [--no-pop] [--no-long] [--no-layer] [--no-model]
 """
 import argparse
 import json
@@ -21,8 +22,39 @@ for p in (ROOT, os.path.join(ROOT, "flash-pop_amd"), os.path.join(ROOT, "tests")
 
 CHUNK = 64
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
-TRAFFIC_PER_PASS = 474.1e6   # (2 x 543.2 MB single passes + 809.9 MB for the dk + dv launch) / 4
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+SPIN_UP_SECONDS = 0.3        # see spin_up()
+
+
+def profiled_traffic(kernel):
+    """HBM bytes per launch of `kernel` at config 2 as the hardware counters gave them (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what it reads for a plain copy of known size).  The figure is not
+    measured by this script: it is read from the summary under profiles/ that the counter runs
+    of flash-pop_amd/profile_counters.sh produced, together with the commit it was measured at.
+    -> (bytes or None, commit or None)"""
+    import glob
+    import re
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        with open(path) as f:
+            m = re.search(r"^HBM_TRAFFIC %s bytes_per_launch=(\d+) measured_at=(\w+)" % re.escape(kernel), f.read(), re.M)
+        if m:
+            return int(m.group(1)), m.group(2)
+    return None, None
+
+
+def spin_up(step, seconds=SPIN_UP_SECONDS):
+    """Part of set-up, before the warm-up steps: keeps the device busy with the benchmarked step
+    until its clocks have settled.  From idle the first ~50 steps (~25 ms) of this workload run up
+    to 20 % slower than every later one; a run of `--warmup 5 --steps 20` would time only that ramp."""
+    import torch
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        n += 10
+    return n
 
 
 def algorithmic_flops(B, T, H, dk, dv, C=CHUNK):
@@ -63,6 +95,7 @@ def gpu_leg(args):
             ev[2].record()
         return grads
 
+    spin_steps = spin_up(step, args.spin_up) if args.spin_up > 0 else 0
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -72,32 +105,23 @@ def gpu_leg(args):
         step(events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    # events on the stream the kernels are launched on (torch's current stream): the forward
+    # launch lies between the first two of a step, the backward launch between the last two
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
     ms_per_step = wall * 1e3 / args.steps
 
-    # how fast the device streams a pass's tensors in this layout and access pattern with no staging and no math
-    lib = _lib.load()
-    y_probe = torch.empty_like(v)
-    probe = lambda: lib.fp_probe_stream_pattern(q.data_ptr(), k.data_ptr(), v.data_ptr(), y_probe.data_ptr(), B, T, H, dk, dv,
-                                                torch.cuda.current_stream().cuda_stream)
-    for _ in range(5):
-        probe()
-    pe = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    pe[0].record()
-    for _ in range(20):
-        probe()
-    pe[1].record()
-    torch.cuda.synchronize()
-    stream_ms = pe[0].elapsed_time(pe[1]) / 20
-
     f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
     b_fwd, b_bwd = algorithmic_bytes(B, T, H, dk, dv)
     tflops = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
-    # one step = 4 passes of the same kernel body in 3 launches: forward, dq, and dk + dv sharing a launch
-    passes, launches = 4, 3
-    avg_pass_ms = (fwd_ms + bwd_ms) / passes
-    achieved_gbs = (b_fwd + b_bwd) / passes / (avg_pass_ms * 1e-3) / 1e9
+    # A step is two launches: the forward pass and the whole backward in one kernel, which is the
+    # dominant one (about 70 % of the step).  Its roofline: the bytes the backward has to move
+    # (q, k, v, dO in; dq, dk, dv out, each once) over its launch duration.
+    bwd_kernel = "retention_bwd_fused_kernel"
+    bwd_gbs = b_bwd / (bwd_ms * 1e-3) / 1e9
+    fwd_gbs = b_fwd / (fwd_ms * 1e-3) / 1e9
+    step_gbs = (b_fwd + b_bwd) / (ms_per_step * 1e-3) / 1e9
+    traffic, traffic_commit = profiled_traffic(bwd_kernel)
 
     out = {
         "metric": "fwd+bwd retention TFLOP/s, B=8 H=16 T=4096 d=128 bf16",
@@ -119,28 +143,29 @@ def gpu_leg(args):
         "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         # the same time priced with only the causal half of every C x C tile counted (C -> (C + 1) / 2)
         "tflops_causal_only": round(sum(algorithmic_flops(B, T, H, dk, dv, C=(CHUNK + 1) / 2)) / (ms_per_step * 1e-3) / 1e12, 2),
+        "set_up": {"spin_up_seconds": args.spin_up, "spin_up_steps": spin_steps,
+                   "why": "device clocks settle over the first ~50 steps from idle; set-up ends with this much of the "
+                          "same work, then the --warmup steps, then the timed --steps"},
         "roofline": {
             "bound": "hbm",
-            "kernel": "retention_pass_ws_kernel<128, 0, 1> (forward, dq) and retention_pass_multi_kernel<128, 0, 1> "
-                      "(dk and dv passes in one launch)",
-            "achieved": round(achieved_gbs, 1),
+            "kernel": bwd_kernel + " (one launch = the whole backward of a step: dq, dk, dv)",
+            "achieved": round(bwd_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
-            # HBM bytes per pass from FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy
-            # (profiles/retention_pass_ws_kernel_128_config2.md); the same for every run of this shape
-            "traffic": TRAFFIC_PER_PASS,
-            "passes_per_step": passes,
-            "launches_per_step": launches,
-            "avg_pass_ms": round(avg_pass_ms, 4),
-            "algorithmic_bytes_per_pass": (b_fwd + b_bwd) // passes,
-            # the forward launch on its own: one launch of retention_pass_ws_kernel<128, 0, 1>
+            "frac": round(bwd_gbs / HBM_PEAK_GBS, 4),
+            "traffic": traffic,
+            "traffic_measured_at_commit": traffic_commit,
+            "launch_ms": round(bwd_ms, 4),
+            "algorithmic_bytes_per_launch": b_bwd,
+            # the other launch of a step and the step as a whole, priced the same way
+            "forward_kernel": "retention_pass_ws_kernel<128, 0, 1>",
             "forward_launch_ms": round(fwd_ms, 4),
-            "forward_launch_algorithmic_gbs": round(b_fwd / (fwd_ms * 1e-3) / 1e9, 1),
-            # fp_probe_stream_pattern: the forward pass's loads and stores alone, same grid and placement
-            "stream_floor_ms": round(stream_ms, 4),
-            "stream_floor_gbs": round(b_fwd / (stream_ms * 1e-3) / 1e9, 1),
-            "forward_launch_vs_stream_floor": round(stream_ms / fwd_ms, 3),
+            "forward_algorithmic_bytes_per_launch": b_fwd,
+            "forward_achieved": round(fwd_gbs, 1),
+            "forward_frac": round(fwd_gbs / HBM_PEAK_GBS, 4),
+            "step_algorithmic_bytes": b_fwd + b_bwd,
+            "step_achieved": round(step_gbs, 1),
+            "step_frac": round(step_gbs / HBM_PEAK_GBS, 4),
         },
     }
 
@@ -359,15 +384,17 @@ def model_leg(args, dev):
     }
 
 
-def cpu_leg(sample_batch=8, reps=2):
+def cpu_leg(sample_batch=8, reps=3):
     """The oracle (chunk 64, fp32, torch autograd for the backward) on the host cores, on
-    `sample_batch` of the 8 sequences of config 2."""
+    `sample_batch` of the 8 sequences of config 2.  Threads: what torch takes from the
+    environment (OMP_NUM_THREADS, else every core the process may run on)."""
     import torch
     import oracle
     import helpers as hp
 
-    threads = min(16, os.cpu_count() or 1)
-    torch.set_num_threads(threads)
+    allowed = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    if "OMP_NUM_THREADS" not in os.environ:
+        torch.set_num_threads(allowed)
     B, T, H, dk, dv = sample_batch, 4096, 16, 128, 128
     decays = oracle.head_decays(H)
     q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0)
@@ -384,6 +411,9 @@ def cpu_leg(sample_batch=8, reps=2):
         "value": round((f_fwd + f_bwd) / sec / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
+        "host_cores": os.cpu_count(),
+        "cores_allowed": allowed,
+        "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
         "kind": "port",
         "sample": f"{B} of the 8 sequences of config 2 (H=16 T=4096 d=128), fp32, chunk 64, fwd+bwd, "
                   f"median of {reps} after 1 warm-up, {sec:.2f} s each",
@@ -396,6 +426,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--spin-up", type=float, default=SPIN_UP_SECONDS,
+                    help="seconds of the benchmarked step run during set-up so that the device clocks have settled (0: none)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
     ap.add_argument("--no-long", action="store_true", help="skip the long-context (config 3) timing")

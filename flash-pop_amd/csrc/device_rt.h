@@ -74,28 +74,4 @@ FP_DEVICE u32x2 buf_load64(BufView b, uint32_t off) { return __builtin_amdgcn_ra
 FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, b.rsrc, off, 0, 0); }
 FP_DEVICE void buf_store64(BufView b, uint32_t off, u32x2 v) { __builtin_amdgcn_raw_buffer_store_b64(v, b.rsrc, off, 0, 0); }
 
-// Optional instrumentation for profiling builds only.
-//   -DFPK_DBGFLAGS : run-time switches that disable parts of the kernel (timing experiments)
-//   -DFPK_PROFILE  : timeline stamps; slot k of iteration `it` records the shader clock for
-//                    lane 0 of the calling wave of workgroup 0 (perturbs the timing noticeably)
-#ifdef FPK_DBGFLAGS
-__device__ int g_dbg_flags = 0;   // 1 no global loads, 2 readout waves idle, 4 state waves idle
-FP_DEVICE int dbg_flags() { return g_dbg_flags; }
-#else
-FP_DEVICE int dbg_flags() { return 0; }
-#endif
-#ifdef FPK_PROFILE
-__device__ unsigned long long* g_prof_buf = nullptr;
-FP_DEVICE void prof_stamp(int it, int slot) {
-  __builtin_amdgcn_sched_barrier(0);
-  if (g_prof_buf && blockIdx.x == 0 && (threadIdx.x & 63) == 0 && it < 64) {
-    const int wave = threadIdx.x >> 6;
-    g_prof_buf[(wave * 64 + it) * 8 + slot] = __builtin_amdgcn_s_memtime();
-  }
-  __builtin_amdgcn_sched_barrier(0);
-}
-#else
-FP_DEVICE void prof_stamp(int, int) {}
-#endif
-
 }  // namespace fprt

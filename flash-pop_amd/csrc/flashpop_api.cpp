@@ -392,10 +392,9 @@ struct Suffixes {
 
 int check_fused(const Shape& s, int block, int sfx_len) {
   if (block < 1) return fail(FP_ERR_BAD_SHAPE, "block_size must be >= 1 (got %d)", block);
-  if (s.T % block != 0)
-    return fail(FP_ERR_BAD_SHAPE, "the fused POP op needs T to be a multiple of block_size (got T=%d, block_size=%d)", s.T, block);
-  if (sfx_len < 1 || sfx_len > fpk::CH)
-    return fail(FP_ERR_BAD_SHAPE, "suffix length must be in 1..%d (got %d)", fpk::CH, sfx_len);
+  if (sfx_len < 1) return fail(FP_ERR_BAD_SHAPE, "suffix length must be positive (got %d)", sfx_len);
+  if (sfx_len > fpk::CH && (s.dk > 128 || s.dv > 128))
+    return fail(FP_ERR_UNSUPPORTED_DIM, "suffixes longer than %d tokens need dk and dv of 64 or 128 (got %d, %d)", fpk::CH, s.dk, s.dv);
   if ((long long)s.B * (s.T / block + 1) * sfx_len >= (1LL << 32))
     return fail(FP_ERR_BAD_SHAPE, "too many suffix rows: B * (T / block_size + 1) * sfx_len must stay below 2^32");
   return FP_OK;
@@ -685,20 +684,6 @@ int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, voi
                             int dv, double eps, void* stream) {
   if (!r || !g || !d_out || !d_r || !d_g) return fail(FP_ERR_NULL_POINTER, "r, g, d_out, d_r and d_g must not be NULL");
   return gated_norm(r, g, d_out, nullptr, d_r, d_g, rows, H, dv, eps, stream);
-}
-
-int fp_probe_stream_pattern(const void* x, const void* w, const void* z, void* y, int B, int T, int H, int dA, int dB,
-                            void* stream) {
-  if (!x || !w || !z || !y) return fail(FP_ERR_NULL_POINTER, "x, w, z and y must not be NULL");
-  if (B < 1 || H < 1 || T < fpk::CH || T % fpk::CH != 0)
-    return fail(FP_ERR_BAD_SHAPE, "B, H >= 1 and T a positive multiple of %d expected (got %d, %d, %d)", fpk::CH, B, H, T);
-  if (dA != 128 || dB < fpk::BV || dB % fpk::BV != 0)
-    return fail(FP_ERR_UNSUPPORTED_DIM, "the probe covers dA = 128 and dB a multiple of %d (got %d, %d)", fpk::BV, dA, dB);
-  if (misaligned(x) || misaligned(w) || misaligned(z) || misaligned(y)) return fail(FP_ERR_BAD_SHAPE, "tensors must be 16-byte aligned");
-  fpk::StreamProbeArgs a{in(x), in(w), in(z), out(y), B, T, H, dA, dB};
-  const char* msg = "";
-  if (fpk_launch_stream_probe(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s", msg);
-  return FP_OK;
 }
 
 const char* fp_last_error(void) { return g_err; }

@@ -7,7 +7,6 @@
 #include "retention_bwd_fused.h"
 #include "decode_step.h"
 #include "layer_ops.h"
-#include "stream_probe.h"
 
 namespace {
 
@@ -58,17 +57,13 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(cons
   fpk::gated_norm_bwd(args);
 }
 
-__global__ __launch_bounds__(fpk::PROBE_THREADS) void stream_probe_kernel(const fpk::StreamProbeArgs args) {
-  fpk::stream_probe(args, fpk::place_workgroup(fprt::block_index(), fprt::grid_size(), 1).wg);
-}
-
 // LDS above 64 KB has to be opted into once per device and kernel.  One bit per kernel (`slot`)
 // and device, shared by all threads of the process: once any thread has run a kernel on a device,
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
-static_assert(2 * fpk::PASS_KERNELS <= 31, "one bit per kernel instantiation, single and paired");
-std::atomic<uint32_t> g_armed[kMaxDevices];
+static_assert(2 * fpk::PASS_KERNELS <= 62, "one bit per kernel instantiation, single and paired");
+std::atomic<uint64_t> g_armed[kMaxDevices];
 
 template <typename Kernel, typename... More>
 int launch(Kernel kernel, int threads, int lds, int slot, int passes, hipStream_t stream, const char** err,
@@ -79,14 +74,14 @@ int launch(Kernel kernel, int threads, int lds, int slot, int passes, hipStream_
     return 1;
   }
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1u << slot))) {
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1ull << slot))) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
         hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(1u << slot, std::memory_order_release);
+    if (tracked) g_armed[dev].fetch_or(1ull << slot, std::memory_order_release);
   }
   const int nwg = a.slots * a.H * (a.dB / fpk::BV) * passes;
   hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a, more...);
@@ -100,16 +95,6 @@ int launch(Kernel kernel, int threads, int lds, int slot, int passes, hipStream_
 
 }  // namespace
 
-#ifdef FPK_PROFILE
-extern "C" int fpk_prof_set(void* buf) {
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fprt::g_prof_buf), &buf, sizeof buf);
-}
-#endif
-#ifdef FPK_DBGFLAGS
-extern "C" int fpk_dbg_set(int flags) {
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fprt::g_dbg_flags), &flags, sizeof flags);
-}
-#endif
 
 // ---- scratch memory that no call allocates ------------------------------------------------------
 // fp_retention_fwd_split_static runs the split-sequence forward without a workspace from the
@@ -217,16 +202,16 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* stream, const char** 
     *err = "hipGetDevice failed";
     return 1;
   }
-  // the opt-in to more than 64 KB of LDS, once per device (bit 31 of the per-device word)
+  // the opt-in to more than 64 KB of LDS, once per device (the top bit of the per-device word)
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1u << 31))) {
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1ull << 63))) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(retention_bwd_fused_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, fpk::fb_lds_bytes()) != hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(1u << 31, std::memory_order_release);
+    if (tracked) g_armed[dev].fetch_or(1ull << 63, std::memory_order_release);
   }
   hipLaunchKernelGGL(retention_bwd_fused_kernel, dim3((unsigned)(2 * a.B * a.H)), dim3(fpk::FB_THREADS), fpk::fb_lds_bytes(),
                      static_cast<hipStream_t>(stream), a);
@@ -311,16 +296,5 @@ int fpk_launch_gated_norm(const fpk::GatedNormArgs& a, void* stream, const char*
   else
     hipLaunchKernelGGL(gated_norm_bwd_kernel, dim3((unsigned)blocks), dim3(fpk::LAYER_THREADS), 0,
                        static_cast<hipStream_t>(stream), a);
-  return launched(err);
-}
-
-int fpk_launch_stream_probe(const fpk::StreamProbeArgs& a, void* stream, const char** err) {
-  long long blocks = 0;
-  if (const char* why = fpk::plan_stream_probe(a, blocks)) {
-    *err = why;
-    return 1;
-  }
-  hipLaunchKernelGGL(stream_probe_kernel, dim3((unsigned)blocks), dim3(fpk::PROBE_THREADS), 0,
-                     static_cast<hipStream_t>(stream), a);
   return launched(err);
 }

@@ -34,7 +34,8 @@ struct PassArgs {
   uint16_t* Bout;        // R after every full block, [B, nblk, H, dk*dv], nullable (forward only)
   const uint16_t* Bin;   // added to R before the chunk that ends each full block, nullable (reverse only)
   // Suffix tensors, [B, nblk + 1, Ls, H, d] in the roles of X, W, Z, Y (all four or none; Ls > 0
-  // selects the suffix walk, which needs T == nblk * block).
+  // selects the suffix walk).  Tokens after the last block boundary are walked like any others;
+  // Rout (forward) and R0 (reverse) then belong to the state at that boundary, nblk * block.
   const uint16_t* Xs;
   const uint16_t* Ws;
   const uint16_t* Zs;
@@ -44,7 +45,7 @@ struct PassArgs {
   int nblk;              // number of full blocks (T / block), 0 if block == 0
   int block;             // block size in tokens; chunks never straddle a multiple of it (0: none)
   int reverse;
-  int Ls;                // tokens per suffix, 1..CH; 0: no suffixes
+  int Ls;                // tokens per suffix (walked in parts of CH); 0: no suffixes
   int state_only;        // only R is wanted (Rout per sequence): X is not read, Y not written, no read-out
   int slots;             // workgroups per (head, column tile); workgroup `slot` walks the batch entries
                          // slot, slot + slots, ... one after another.  0: the launcher chooses.
@@ -165,15 +166,6 @@ struct GatedNormArgs {
 };
 constexpr int LAYER_THREADS = 256;
 
-// The access pattern of one pass and nothing else (stream_probe.h): X, W [B,T,H,dA] read, the Z
-// tiles [B,T,H,dB] copied to Y.  T a multiple of 64, dA = 128, dB a multiple of 64.
-struct StreamProbeArgs {
-  const uint16_t *X, *W, *Z;
-  uint16_t* Y;
-  int B, T, H, dA, dB;
-};
-constexpr int PROBE_THREADS = 512;
-
 }  // namespace fpk
 
 // Launches the pass kernel on `stream` (a hipStream_t, or ignored by the CPU test harness).
@@ -210,6 +202,3 @@ int fpk_launch_decode(const fpk::DecodeArgs& args, void* stream, const char** er
 // Launch the rotary kernel / the gated per-head normalisation (forward if a.out, else backward).
 int fpk_launch_rotary(const fpk::RotaryArgs& args, void* stream, const char** err);
 int fpk_launch_gated_norm(const fpk::GatedNormArgs& args, void* stream, const char** err);
-
-// Launches the access-pattern probe (see stream_probe.h).  Same conventions as fpk_launch_pass.
-int fpk_launch_stream_probe(const fpk::StreamProbeArgs& args, void* stream, const char** err);

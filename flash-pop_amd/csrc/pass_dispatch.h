@@ -9,7 +9,7 @@
 namespace fpk {
 
 // Number of kernel instantiations `dispatch_pass` can pick from (its `slot` argument is below this).
-constexpr int PASS_KERNELS = 14;
+constexpr int PASS_KERNELS = 17;
 
 // Checks what the walks assume about `a` and chooses a.slots (workgroups per (head, column tile))
 // for a device with `compute_units` units.  Returns nullptr, or a message for the caller.
@@ -21,8 +21,9 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
   if (a.dB < BV || a.dB % BV != 0) return "dB must be a multiple of 64";
   if (suffix) {
     // the C-ABI layer reports these to the caller in its own words
-    if (blocks || a.block <= 0 || a.T != a.nblk * a.block || a.Ls > CH || !a.Xs || !a.Ws || !a.Zs || !a.Ys)
-      return "suffix walk: needs T == nblk * block, 1 <= Ls <= 64 and all four suffix tensors";
+    if (blocks || a.block <= 0 || a.nblk != a.T / a.block || !a.Xs || !a.Ws || !a.Zs || !a.Ys)
+      return "suffix walk: needs nblk == T / block and all four suffix tensors";
+    if (a.Ls > CH && !narrow) return "suffixes longer than 64 tokens need dk and dv of 64 or 128";
     a.slots = a.B;
   }
   // One workgroup per (batch entry, head, column tile) while that fits the chip once; beyond that
@@ -88,7 +89,10 @@ template <typename Run>
 int dispatch_pass(const PassArgs& a, Run&& run) {
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool suffix = a.Ls > 0, multi = a.slots < a.B;
+  // trailing tokens after the last block boundary, or suffixes in several parts: the general suffix walk
+  const bool suffix_any = suffix && (a.T != a.nblk * a.block || a.Ls > CH);
   if (a.dA == 64) {
+    if (suffix_any) return run.template go<64, WALK_SUFFIX_ANY, 1>(14);
     if (suffix) return run.template go<64, WALK_SUFFIX, 1>(0);
     if (blocks) return run.template go<64, WALK_BLOCKS, 1>(1);
     if (a.state_only) return run.template go<64, WALK_STATE, 1>(2);
@@ -96,6 +100,7 @@ int dispatch_pass(const PassArgs& a, Run&& run) {
     return run.template go<64, WALK_PLAIN, 1>(4);
   }
   if (a.dA == 128) {
+    if (suffix_any) return run.template go<128, WALK_SUFFIX_ANY, 1>(15);
     if (suffix) return run.template go<128, WALK_SUFFIX, 1>(5);
     if (blocks) return run.template go<128, WALK_BLOCKS, 1>(6);
     if (a.state_only) return run.template go<128, WALK_STATE, 1>(7);
@@ -103,6 +108,7 @@ int dispatch_pass(const PassArgs& a, Run&& run) {
     return run.template go<128, WALK_PLAIN, 1>(9);
   }
   // dA = 256: two visits per chunk, 128 of the 256 contraction columns each
+  if (suffix_any) return run.template go<128, WALK_SUFFIX_ANY, 2>(16);
   if (suffix) return run.template go<128, WALK_SUFFIX, 2>(12);
   if (a.state_only) return run.template go<128, WALK_STATE, 2>(13);
   if (blocks) return run.template go<128, WALK_BLOCKS, 2>(10);

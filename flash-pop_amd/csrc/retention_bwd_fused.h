@@ -130,12 +130,6 @@ FP_DEVICE Common make_common(const FusedBwdArgs& p, int stream) {
 // view of the rows of chunk `ci` of one tensor for this stream; rows past the sequence read as
 // zero and are dropped on stores
 FP_DEVICE fprt::BufView chunk_view(const Common& k, const void* base, int ci, bool store = false) {
-#ifdef FB_NOLOAD
-  if (!store) ci = -1;
-#endif
-#ifdef FB_NOSTORE
-  if (store) ci = -1;
-#endif
   const bool ok = ci >= 0 && ci < k.nch;
   const int t0 = ok ? ci * CH : 0;
   const int L = ok ? (k.T - t0 < CH ? k.T - t0 : CH) : 0;
@@ -363,7 +357,6 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
 
   for (int ci = k.nch - 1; ci >= 0; --ci) {
     const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
-    fprt::prof_stamp(k.nch - 1 - ci, 0);
     // ---- the previous chunk's outputs leave (nothing writes the staging tiles before the next barrier)
     if (ci < k.nch - 1) {
       drain_tile(k, OUT, p.dv, ci + 1);
@@ -421,9 +414,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       acc[0][r] *= wread0;
       acc[1][r] *= wread1;
     }
-    fprt::prof_stamp(k.nch - 1 - ci, 1);
     fprt::block_sync();
-    fprt::prof_stamp(k.nch - 1 - ci, 2);
 
     // ---- stretch 2: Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]
     {
@@ -477,20 +468,16 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
         fprt::sched_fence();
       }
     }
-    fprt::prof_stamp(k.nch - 1 - ci, 3);
     // nobody reads this chunk's k and v tiles or the old copy of dS any more
     stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
     load_tiles<2>(k, src_kv, ci - 2, pf_kv);
 #pragma unroll
     for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
-    fprt::prof_stamp(k.nch - 1 - ci, 4);
     fprt::block_sync();
-    fprt::prof_stamp(k.nch - 1 - ci, 5);
 
     // ---- stretch 3: every read of this chunk's q and dO tiles is done
     stage_tiles<2>(k, TL, pf_qg);
     load_tiles<2>(k, src_qg, ci - 2, pf_qg);
-    fprt::prof_stamp(k.nch - 1 - ci, 6);
     fprt::block_sync();
   }
   drain_tile(k, OUT, p.dv, 0);
@@ -713,9 +700,6 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
 // launch index -> kind and stream: the reverse workgroups (the longer ones) come first
 FP_DEVICE void fused_bwd(const FusedBwdArgs& p, char* lds, int block) {
   const int streams = p.B * p.H;
-#ifdef FB_ONLY
-  if ((block < streams) != (FB_ONLY == 0)) return;
-#endif
   if (block < streams) {
     if (fprt::thread_index() < 256) fused_bwd_reverse<0>(p, lds, block);
     else fused_bwd_reverse<1>(p, lds, block);

@@ -67,15 +67,19 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 // WALK_BLOCKS  the pass writes block states (Bout) or reads their gradients (Bin);
 // WALK_MULTI   a workgroup walks several batch entries (p.slots < p.B), so that short sequences
 //              keep the load pipeline full across sequence boundaries;
-// WALK_SUFFIX  a suffix of p.Ls tokens hangs off every block boundary (positions 0, block, ...,
-//              T; T is a multiple of the block size).  It is one more item of the walk, placed at
+// WALK_SUFFIX  a suffix of p.Ls <= CH tokens hangs off every block boundary (positions 0, block,
+//              ..., T; T is a multiple of the block size).  It is one more item of the walk, placed at
 //              its boundary, with its own tensors: it reads the state at the boundary without
 //              advancing it.  Walking forward its keys stay out of R and R is not decayed; walking
 //              backward its read-out weight is 0 and what it adds to R (the gradient of the state
 //              it read) is not decayed either.
+// WALK_SUFFIX_ANY  the same for any T and any p.Ls: tokens after the last block boundary are
+//              walked as context with no suffix behind them (Rout, forward, and R0, backward,
+//              then belong to the state at that boundary), and a suffix of more than CH tokens
+//              is walked in parts on a copy of the state.
 // WALK_STATE   like WALK_MULTI, but only the final R of every sequence is wanted (p.state_only):
 //              the readout waves feed Z and do nothing else, X is not read and Y not written.
-enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WALK_STATE = 4 };
+enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WALK_STATE = 4, WALK_SUFFIX_ANY = 5 };
 
 // NH = 2 handles a contraction width of 2 DA (p.dA = 256 with DA = 128) with the LDS footprint of
 // DA: every chunk is visited twice, once per half of the columns of X and W (of the rows of R).
@@ -91,7 +95,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   static_assert(DA == 64 || DA == 128, "wave-specialised pass: dA must be 64 or 128");
   static_assert(NH == 1 || MODE != WALK_MULTI, "two halves: not with several sequences per workgroup and a read-out");
   constexpr bool STATE = MODE == WALK_STATE;
-  constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI || STATE, SFX = MODE == WALK_SUFFIX;
+  constexpr bool BLOCKS = MODE == WALK_BLOCKS, MULTI = MODE == WALK_MULTI || STATE;
+  constexpr bool SFX_ANY = MODE == WALK_SUFFIX_ANY, SFX = MODE == WALK_SUFFIX || SFX_ANY;
   constexpr int X_LD = DA + 8;
   constexpr int T_LD = CH + 4;      // row length of the transposed tiles (tokens)
   constexpr int RT_LD = DA + 8;
@@ -120,7 +125,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   const int h = (wg / ntile) % p.H;
   const int slot = (wg / ntile) / p.H;   // first batch entry of this workgroup
 
-  const int dbg = fprt::dbg_flags();   // always 0 outside profiling builds
   const int T = p.T;
   const int bs = (BLOCKS || SFX) ? p.block : 0;   // only these walks cut chunks at block boundaries
   const bool rev = io.reverse != 0;
@@ -156,22 +160,37 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     bool ok, first, last;   // exists / first item of its sequence / last item of its sequence
     bool sfx;               // a suffix (t0 is its block boundary) rather than a context chunk
     int n;                  // WALK_SUFFIX only: index of the suffix, or of the context chunk's block
+    int part;               // WALK_SUFFIX only: which CH tokens of a suffix longer than a chunk (0 otherwise)
     int h;                  // NH = 2 only: which half of the contraction this visit covers
     uint32_t row;           // index of the item's first row among all rows of its tensor
   };
-  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0, 0, 0u};
+  const Chunk no_chunk = {0, 0, 0, false, false, false, false, 0, 0, 0, 0u};
+  // A suffix of more than CH tokens is walked in parts of CH tokens (the last one shorter), in
+  // walking order; between its parts the state moves on as between context chunks, on a copy.
+  const int sfx_parts = SFX_ANY ? (p.Ls + CH - 1) / CH : 1;
+  auto part_len = [&](int part) { return p.Ls - CH * part < CH ? p.Ls - CH * part : CH; };
   auto with_row = [&](Chunk ck) {
-    ck.row = (SFX && ck.sfx) ? ((uint32_t)ck.b * (p.nblk + 1) + ck.n) * p.Ls : (uint32_t)ck.b * T + ck.t0;
+    ck.row = (SFX && ck.sfx) ? ((uint32_t)ck.b * (p.nblk + 1) + ck.n) * p.Ls + CH * ck.part : (uint32_t)ck.b * T + ck.t0;
     return ck;
   };
+  // the part of suffix n at boundary `pos` that the walk meets first
+  auto enter_suffix = [&](Chunk& ck, int n, int pos, bool ends_walk) {
+    ck.sfx = true;
+    ck.n = n;
+    ck.t0 = pos;
+    ck.part = rev ? sfx_parts - 1 : 0;
+    ck.L = part_len(ck.part);
+    ck.last = ends_walk && sfx_parts == 1;
+  };
   auto first_chunk = [&](int b) {
-    Chunk ck = {b, 0, 0, b < p.B, true, false, false, 0};
+    Chunk ck = {b, 0, 0, b < p.B, true, false, false, 0, 0};
     if (ck.ok) {
-      if (SFX) {   // the suffix at the first boundary met: position 0, or T walking backward
-        ck.sfx = true;
-        ck.n = rev ? p.nblk : 0;
-        ck.t0 = rev ? T : 0;
-        ck.L = p.Ls;
+      if (SFX_ANY && rev && T > p.nblk * bs) {   // tokens after the last boundary: the walk back starts with them
+        ck.n = p.nblk;
+        ck.t0 = T - CH > p.nblk * bs ? T - CH : p.nblk * bs;
+        ck.L = T - ck.t0;
+      } else if (SFX) {   // the suffix at the first boundary met: position 0, or T walking backward
+        enter_suffix(ck, rev ? p.nblk : 0, rev ? T : 0, false);
       } else {
         chunk_at(rev ? T : 0, ck.t0, ck.L);
         ck.last = !has_more(next_pos(ck.t0, ck.L));
@@ -188,22 +207,34 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       return again;
     }
     if (ck.last) return MULTI ? first_chunk(ck.b + p.slots) : no_chunk;
-    Chunk n = {ck.b, 0, 0, true, false, false, false, 0};
+    Chunk n = {ck.b, 0, 0, true, false, false, false, 0, 0};
+    if (SFX_ANY && ck.sfx && (rev ? ck.part > 0 : ck.part < sfx_parts - 1)) {   // the next part of the same suffix
+      n = ck;
+      n.first = false;
+      n.h = 0;
+      n.part = rev ? ck.part - 1 : ck.part + 1;
+      n.L = part_len(n.part);
+      // the walk ends with the last part of the suffix at position T (forward) or 0 (backward)
+      n.last = (rev ? n.part == 0 && ck.t0 == 0 : n.part == sfx_parts - 1 && ck.t0 == T);
+      return with_row(n);
+    }
     if (SFX) {
-      // Block m spans [m bs, (m + 1) bs).  After a suffix comes the nearest context chunk of the
-      // block that follows it in walking order; after the context chunk that reaches the far
-      // boundary of its block comes that boundary's suffix.
+      // Block m spans [m bs, (m + 1) bs); the tokens after the last boundary, if any, form a
+      // shorter block nblk that ends the walk without a suffix.  After a suffix comes the nearest
+      // context chunk of the block that follows it in walking order; after the context chunk that
+      // reaches the far boundary of its block comes that boundary's suffix.
       if (!rev) {
-        const int m = ck.n, pos = ck.sfx ? ck.t0 : ck.t0 + ck.L, lim = (m + 1) * bs;
+        const int m = ck.n, pos = ck.sfx ? ck.t0 : ck.t0 + ck.L, lim = (!SFX_ANY || (m + 1) * bs < T) ? (m + 1) * bs : T;
         if (!ck.sfx && pos == lim) {
-          n.sfx = true; n.n = m + 1; n.t0 = pos; n.L = p.Ls; n.last = pos == T;
+          enter_suffix(n, m + 1, pos, pos == T);
         } else {
           n.n = m; n.t0 = pos; n.L = (pos + CH < lim ? pos + CH : lim) - pos;
+          n.last = SFX_ANY && m == p.nblk && pos + n.L == T;
         }
       } else {
         const int m = ck.sfx ? ck.n - 1 : ck.n, pos = ck.t0, lo = m * bs;
         if (!ck.sfx && pos == lo) {
-          n.sfx = true; n.n = m; n.t0 = pos; n.L = p.Ls; n.last = pos == 0;
+          enter_suffix(n, m, pos, pos == 0);
         } else {
           n.n = m; n.t0 = pos - CH > lo ? pos - CH : lo; n.L = pos - n.t0;
         }
@@ -292,14 +323,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       u32x2 z[4];
     };
     auto feed_load_x = [&](FeedRegs& fr, const Chunk& c2) {
-      const bool live = c2.ok && !(dbg & 1) && !STATE;
+      const bool live = c2.ok && !STATE;
       const uint32_t lenA = live ? (uint32_t)(c2.L - 1) * rowA + DA * 2 : 0u;
       const fprt::BufView xv = fprt::make_buf(((SFX && c2.sfx) ? Xsg : Xg) + (live ? rowsA(c2) : 0), lenA);
 #pragma unroll
       for (int u = 0; u < NXP; ++u) fr.x[u] = fprt::buf_load128(xv, xg_off[u]);
     };
     auto feed_load_z = [&](FeedRegs& fr, const Chunk& c2) {
-      const bool live = c2.ok && !(dbg & 1);
+      const bool live = c2.ok;
       const uint32_t lenB = live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u;
       const fprt::BufView zv = fprt::make_buf(((SFX && c2.sfx) ? Zsg : Zg) + (live ? rowsB(c2) : 0), lenB);
 #pragma unroll
@@ -372,21 +403,13 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
         int e = L - 1 - i_row;
         if (e < 0) e = 0;
         wread = io.s_read * fprt::exp2_approx((float)e * lg);
-        if (SFX && ck.sfx) wread = 0.f;   // nothing downstream of a suffix reaches back into it
+        // nothing downstream of a suffix reaches back into it: its last tokens meet a zero gradient state
+        if (SFX && ck.sfx && ck.part == sfx_parts - 1) wread = 0.f;
       }
 
-      fprt::prof_stamp(it, 0);
       if (STATE) {   // feed Z for the state waves, nothing else
         feed_store_z(feed, s ^ 1);
         feed_load_z(feed, ck2);
-        fprt::block_sync();
-        ckp = ck;
-        ck = ck1;
-        ck1 = ck2;
-        return ck.ok;
-      }
-      if (dbg & 2) {
-        if (closes) fprt::block_sync();
         fprt::block_sync();
         ckp = ck;
         ck = ck1;
@@ -411,7 +434,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
 #pragma unroll
       for (int t = 0; t < KS; ++t) yacc = fprt::mfma_32x32x16_bf16(rf[t], xf[t], yacc);
       fprt::sched_fence();
-      fprt::prof_stamp(it, 1);
 
       // ---- phase 2: scores^T of this wave's tile; Z arrives meanwhile; X of chunk it + 1 goes
       // to the other stage
@@ -430,7 +452,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       feed_store_x(feed, s ^ 1);
       feed_load_x(feed, ck2);
       fprt::sched_fence();
-      fprt::prof_stamp(it, 2);
 
       // ---- phase 3: the read-out is scaled, P converted and put where the partner wave finds
       // it, and Z of chunk it + 1 is transposed into the other stage.  Accumulator element
@@ -455,7 +476,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       feed_store_z(feed, s ^ 1);
       feed_load_z(feed, ck2);
       fprt::sched_fence();
-      fprt::prof_stamp(it, 3);
       if (!closes) {   // first half of the contraction: nothing to finish yet
         fprt::block_sync();
         ckp = no_chunk;
@@ -490,10 +510,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
         d[1] = fprt::pack_bf16x2(yacc[4 * qd + 2], yacc[4 * qd + 3]);
         st64(yb + y_off + 8 * qd, d);
       }
-      fprt::prof_stamp(it, 4);
 
       fprt::block_sync();
-      fprt::prof_stamp(it, 5);
       ckp = ck;
       ck = ck1;
       ck1 = ck2;
@@ -549,7 +567,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   // same in every iteration; a chunk that does not exist gets zero-length views (no traffic).
   auto prefetch = [&](ChunkRegs& cr, const Chunk& ck) {
     // views that start at the chunk's first row and end with its last: later rows read as zero
-    const bool live = ck.ok && !(dbg & 1);
+    const bool live = ck.ok;
     const uint32_t lenA = live ? (uint32_t)(ck.L - 1) * rowA + DA * 2 : 0u;
     const fprt::BufView wb = fprt::make_buf(((SFX && ck.sfx) ? Wsg : Wg) + (live ? rowsA(ck) : 0), lenA);
 #pragma unroll
@@ -688,7 +706,8 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   int Lk_cached = -1;
   float wkey[4];
   auto store_transposed = [&](const ChunkRegs& cr, const Chunk& ck) {
-    if (SFX && ck.sfx && !rev) return;   // walking forward, a suffix's keys never enter the state
+    // walking forward, a suffix's keys never enter the state (only, on a copy, the state that its own later parts read)
+    if (SFX && ck.sfx && !rev && ck.part == sfx_parts - 1) return;
     if (ck.L != Lk_cached) {
       Lk_cached = ck.L;
 #pragma unroll
@@ -715,6 +734,11 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     }
   };
 
+  // Suffix walk, backward, with tokens after the last block boundary: R0 is the gradient of the
+  // state at that boundary, not at the end of the sequence.  The walk starts from zero and R0 joins
+  // when the boundary is reached, the way block-state gradients do.
+  const bool r0_late = SFX_ANY && rev && io.R0 && T > p.nblk * bs;
+  const bool r0_first = io.R0 && !r0_late;
   // ---- prologue: chunk 0 into stage 0, chunk 1 in flight ----------------------------------
   Chunk cur = first_chunk(slot), nxt = chunk_after(cur);
   prefetch(wregs, cur);
@@ -722,10 +746,10 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   for (int hf = 0; hf < NH; ++hf) {
     // initial R, plus the gradient of the last block state if the first chunk of a reverse pass ends a block
     TileRegs t_init, t_inj;
-    tile_load(t_init, io.R0 ? state_matrix(io.R0, cur.b) : nullptr, true, hf);
+    tile_load(t_init, r0_first ? state_matrix(io.R0, cur.b) : nullptr, true, hf);
     const bool inj = BLOCKS && io.Bin && ends_block(cur.t0 + cur.L);
     tile_load(t_inj, inj ? block_matrix(io.Bin, cur.b, cur.t0 + cur.L) : nullptr, inj, hf);
-    if (io.R0) tile_accumulate(t_init, 0, false, racc[hf]);
+    if (r0_first) tile_accumulate(t_init, 0, false, racc[hf]);
     if (inj) tile_accumulate(t_inj, 0, true, racc[hf]);
   }
   write_rt(0, racc[0]);
@@ -736,6 +760,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
 
   int Lg_cached = -1;
   float gL = 1.f;
+  // suffix walk: R while a suffix in several parts works on its copy (one visit per chunk only:
+  // with two, a second set of both halves does not fit the register file)
+  f32x16 saved[NNW];
   // One iteration: `wregs` holds the W rows of item it + 1 on entry and is reloaded with item
   // it + 2 once they have gone into LDS.  Returns false after the last item.  `half` is the parity
   // of `it` as a type; with NH = 2 it is the half of R this visit updates.
@@ -744,36 +771,38 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     constexpr bool closes = HF == NH - 1;   // the chunk is complete after this visit
     f32x16 (&racc_h)[NNW] = racc[HF];
     const int s = it & 1;
-    fprt::prof_stamp(it, 0);
     const Chunk nn = chunk_after(nxt);
     // gradient of the block state that the next chunk ends (reverse pass); an empty view otherwise
-    const bool inj = BLOCKS && closes && io.Bin && nxt.ok && ends_block(nxt.t0 + nxt.L);
+    // (suffix walk: the gradient of the state at the last boundary, when the next item is that boundary's suffix)
+    const bool inj = closes && nxt.ok && (BLOCKS ? io.Bin && ends_block(nxt.t0 + nxt.L) : r0_late && nxt.sfx && nxt.n == p.nblk && nxt.part == sfx_parts - 1);
     TileRegs t_inj[NH];
-    if (BLOCKS && closes) {
+    if ((BLOCKS || SFX_ANY) && closes) {
+      const uint16_t* const src = !inj ? nullptr : BLOCKS ? block_matrix(io.Bin, nxt.b, nxt.t0 + nxt.L) : state_matrix(io.R0, nxt.b);
 #pragma unroll
-      for (int hf = 0; hf < NH; ++hf) tile_load(t_inj[hf], inj ? block_matrix(io.Bin, nxt.b, nxt.t0 + nxt.L) : nullptr, inj, hf);
+      for (int hf = 0; hf < NH; ++hf) tile_load(t_inj[hf], src, inj, hf);
     }
     // initial state of the next sequence, if the next chunk starts one
     const bool fresh = MULTI && nxt.ok && nxt.first;
     TileRegs t_init;
     if (MULTI) tile_load(t_init, (fresh && io.R0) ? state_matrix(io.R0, nxt.b) : nullptr, fresh, 0);
 
-    if (dbg & 4) {
-      if (!STATE && closes) fprt::block_sync();
-      fprt::block_sync();
-      if (!nxt.ok) return false;
-      cur = nxt;
-      nxt = nn;
-      return true;
-    }
     // A suffix carries tokens only in its first k-steps, and none that enter the state when
     // walking forward: the other k-steps are skipped (uniform branches).
+    // A suffix in several parts works on a copy of the state: R is put aside when the walk
+    // enters the suffix and comes back when it leaves.  Forward, the copy advances through all
+    // parts but the last; backward, it starts from zero and what it holds in the end (the
+    // gradient of the state the suffix read) is added to R.
     const bool sfx_item = SFX && cur.sfx;
-    const int nk = sfx_item ? (rev ? (cur.L + 15) >> 4 : 0) : 4;
+    const bool sfx_multi = SFX_ANY && NH == 1 && sfx_item && sfx_parts > 1;
+    const bool enters = sfx_multi && cur.part == (rev ? sfx_parts - 1 : 0);
+    const bool leaves_sfx = sfx_multi && cur.part == (rev ? 0 : sfx_parts - 1);
+    const bool advances = !sfx_item || rev || cur.part < sfx_parts - 1;
+    const bool decays = !sfx_item || (sfx_multi && (rev ? !enters : advances));
+    const int nk = !sfx_item ? 4 : rev ? (cur.L + 15) >> 4 : advances ? 4 : 0;
 
     // ---- phase 0: request the operands of the state update (this wave's whole W^T slab, the
     // first half of Z^T); decay R while they arrive
-    const int gkey = sfx_item ? 0 : cur.L;   // a suffix does not advance the state
+    const int gkey = decays ? cur.L : 0;   // a suffix in one part does not advance the state
     if (gkey != Lg_cached) {
       Lg_cached = gkey;
       gL = fprt::exp2_approx((float)gkey * lg);
@@ -791,7 +820,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
         for (int nq = 0; nq < NNW; ++nq) zlo[nq][kt] = ld_token_frag(zt + (32 * (nb0 + nq) + c) * T_LD + 16 * kt + 4 * g);
       }
     }
-    if (!sfx_item) {
+    if (SFX_ANY && enters) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq) {
+        saved[nq] = racc_h[nq];
+        if (rev) racc_h[nq] = f32x16{0};
+      }
+    }
+    if (decays) {
 #pragma unroll
       for (int nq = 0; nq < NNW; ++nq) {
 #pragma unroll
@@ -799,7 +835,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       }
     }
     fprt::sched_fence();
-    fprt::prof_stamp(it, 1);
 
     // ---- phase 1: first half of R = gamma^L R + (wkey W)^T Z; in its shadow the rest of Z^T is
     // requested and the W of chunk it + 1 (zeros if there is none) is transposed.  The W^T slab is overwritten only after all of it was read.
@@ -820,7 +855,6 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     }
     store_transposed(wregs, nxt);
     fprt::sched_fence();
-    fprt::prof_stamp(it, 2);
     if (!STATE && closes) fprt::block_sync();   // the readout waves hand their P tiles to each other here
 
     // ---- phase 2: second half of the state update; the row-major copies go out in its shadow
@@ -840,15 +874,24 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     // over, and the bf16 copy for the next chunk's read-out is written.  All of them use this
     // wave's part of the other stage's R buffer, in this order.
     const int t1 = cur.t0 + cur.L;
+    if (SFX_ANY && leaves_sfx) {
+#pragma unroll
+      for (int nq = 0; nq < NNW; ++nq) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) racc_h[nq][r] = rev ? racc_h[nq][r] + saved[nq][r] : saved[nq][r];
+      }
+    }
     if (closes) {
 #pragma unroll
       for (int hf = 0; hf < NH; ++hf) {
         if (BLOCKS && io.Bout && ends_block(t1))
           tile_store(const_cast<uint16_t*>(block_matrix(io.Bout, cur.b, t1)), s ^ 1, racc[hf], hf);
-        if (cur.last && io.Rout) tile_store(const_cast<uint16_t*>(state_matrix(io.Rout, cur.b)), s ^ 1, racc[hf], hf);
+        // the state that leaves: after the last item; walking forward with suffixes, the one that the
+        // suffix at the last block boundary reads (tokens after that boundary are not in it)
+        const bool leaves = (SFX && !rev) ? cur.sfx && cur.n == p.nblk && cur.part == sfx_parts - 1 : cur.last;
+        if (leaves && io.Rout) tile_store(const_cast<uint16_t*>(state_matrix(io.Rout, cur.b)), s ^ 1, racc[hf], hf);
       }
     }
-    fprt::prof_stamp(it, 3);
     if (nxt.ok) {
       if (MULTI && fresh) {
         if (io.R0) {
@@ -858,16 +901,14 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
           for (int nq = 0; nq < NNW; ++nq) racc[0][nq] = f32x16{0};
         }
       }
-      if (BLOCKS && closes && inj) {
+      if ((BLOCKS || SFX_ANY) && closes && inj) {
 #pragma unroll
         for (int hf = 0; hf < NH; ++hf) tile_accumulate(t_inj[hf], s ^ 1, true, racc[hf]);
       }
       // the next visit reads the other half (NH = 2), which this visit did not touch
       if (!STATE) write_rt(s ^ 1, racc[(HF + 1) % NH]);
     }
-    fprt::prof_stamp(it, 4);
     fprt::block_sync();
-    fprt::prof_stamp(it, 5);
     if (!nxt.ok) return false;
     cur = nxt;
     nxt = nn;

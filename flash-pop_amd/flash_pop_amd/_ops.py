@@ -136,8 +136,6 @@ def prepare_suffixes(q_sfx, k_sfx, v_sfx, shape, block_size):
     """Checks of the suffix batch as POPDecoderLayer._suffixes_forward makes them
     (flash_pop/pop_retnet.py:154-159): one suffix per block boundary, N + 1 per sequence."""
     B, T, H, dk, dv = shape
-    if T % block_size != 0:
-        raise ValueError(f"the fused POP op needs T ({T}) to be a multiple of block_size ({block_size})")
     n = B * (T // block_size + 1)
     if q_sfx.dim() != 4 or k_sfx.shape != q_sfx.shape or v_sfx.dim() != 4 or v_sfx.shape[:3] != q_sfx.shape[:3]:
         raise ValueError("expected q_sfx, k_sfx [B*(N+1),Ls,H,dk] and v_sfx [B*(N+1),Ls,H,dv]")

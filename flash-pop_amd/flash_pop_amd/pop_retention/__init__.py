@@ -13,8 +13,9 @@ One POP layer step in a single walk: what POPDecoderLayer.pop_forward obtains fr
 flash_pop_retention followed by fused_chunk_retention on the suffix batch seeded with
 [s, block_states] (flash_pop/pop_retnet.py:107-171), without writing the block states, reading
 them back or concatenating them.  q_sfx, k_sfx, v_sfx are [B * (N + 1), Ls, H, d] with the block
-index fastest (N = T // block_size, T a multiple of block_size, Ls <= 64); last_state is the
-state after the last block, the reference's `states[:, -1]`.
+index fastest (N = T // block_size, any Ls >= 1); last_state is the state after the last full
+block, the reference's `states[:, -1]`.  Tokens after the last block boundary (T % block_size of
+them) are context like any others; no suffix follows them.
 """
 import torch
 

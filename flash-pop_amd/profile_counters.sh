@@ -2,8 +2,8 @@
 # Collects the rocprofv3 evidence for the pass kernels on benchmark configurations 2 and 4 (run from the repo
 # root on a GPU box): kernel-trace statistics, then hardware counters in separate passes (one
 # counter group per run), then the same HBM counters on a plain copy of known size for scaling.
-# Raw output goes to the directory given as the first argument; the figures are summarised by
-# hand into profiles/.
+# Raw output goes to the directory given as the first argument; flash-pop_amd/profile_summary.py turns
+# it into the tables kept under profiles/.
 #   usage: flash-pop_amd/profile_counters.sh <output directory>
 set -e
 R=$(cd "$(dirname "$0")/.." && pwd)
@@ -11,7 +11,7 @@ R=$(cd "$(dirname "$0")/.." && pwd)
 mkdir -p "$1"
 O=$(cd "$1" && pwd)
 cd /tmp && export TMPDIR=/tmp
-BENCH="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu --no-long --no-model"
+BENCH="python3 $R/bench.py --steps 8 --warmup 4 --spin-up 0 --no-cpu --no-long --no-model"
 COPY="python3 $R/bench.py --copy-calibration"
 run() { name=$1; shift; timeout -s KILL 120 rocprofv3 "$@" --output-format csv -d "$O/$name" -o r -- $CMD > "$O/$name.log" 2>&1; }
 CMD=$BENCH run trace --kernel-trace --stats

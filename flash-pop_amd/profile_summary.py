@@ -1,0 +1,100 @@
+"""Turns the raw rocprofv3 output of profile_counters.sh into the tables kept under profiles/.
+
+    python flash-pop_amd/profile_summary.py <output directory of profile_counters.sh> [commit]
+
+Prints markdown: per-kernel durations from the kernel trace, HBM bytes per launch from
+FETCH_SIZE / WRITE_SIZE (KiB per dispatch, each scaled by what the same counter reads for the
+plain 1 GiB copy of `bench.py --copy-calibration`), the shader counters per launch, and one
+`HBM_TRAFFIC <kernel> bytes_per_launch=<n> measured_at=<commit>` line per library kernel, which
+bench.py reads back for the `traffic` field of its roofline object.
+"""
+import csv
+import os
+import re
+import subprocess
+import sys
+from collections import defaultdict
+
+OURS = ("retention_", "segment_scan", "decode_step", "rotary_qk", "gated_norm")
+COPY_KIB = 1 << 20   # the calibration copies 1 GiB
+
+
+def short(name):
+    name = re.sub(r"^void ", "", name).replace("(anonymous namespace)::", "")
+    return re.sub(r"\(.*\)$", "", name)
+
+
+def kernel_stats(path):
+    rows = []
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            if any(k in r["Name"] for k in OURS):
+                rows.append((short(r["Name"]), int(r["Calls"]), float(r["AverageNs"]) / 1e3, int(r["MinNs"]) / 1e3,
+                             int(r["MaxNs"]) / 1e3))
+    return sorted(rows, key=lambda r: -r[1] * r[2])
+
+
+def counters(path):
+    """-> {kernel: {counter: (mean value per dispatch, dispatches)}}"""
+    acc = defaultdict(lambda: defaultdict(list))
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            acc[short(r["Kernel_Name"])][r["Counter_Name"]].append(float(r["Counter_Value"]))
+    return {k: {c: (sum(v) / len(v), len(v)) for c, v in cs.items()} for k, cs in acc.items()}
+
+
+def copy_reading(path, counter):
+    """The counter's largest per-dispatch value in the calibration run: the 1 GiB copy kernel."""
+    best = 0.0
+    for cs in counters(path).values():
+        if counter in cs:
+            best = max(best, cs[counter][0])
+    return best
+
+
+def main():
+    out = sys.argv[1]
+    commit = sys.argv[2] if len(sys.argv) > 2 else subprocess.run(
+        ["git", "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip() or "unknown"
+    p = lambda *a: os.path.join(out, *a)
+
+    print("## Kernel trace (--kernel-trace --stats)\n")
+    print("| kernel | calls | average | min | max |\n|---|---|---|---|---|")
+    for name, calls, avg, lo, hi in kernel_stats(p("trace", "r_kernel_stats.csv")):
+        print(f"| {name} | {calls} | {avg:.1f} us | {lo:.1f} us | {hi:.1f} us |")
+
+    if os.path.exists(p("fetch", "r_counter_collection.csv")):
+        fetch, write = counters(p("fetch", "r_counter_collection.csv")), counters(p("write", "r_counter_collection.csv"))
+        cf, cw = copy_reading(p("copy_fetch", "r_counter_collection.csv"), "FETCH_SIZE"), copy_reading(
+            p("copy_write", "r_counter_collection.csv"), "WRITE_SIZE")
+        sf, sw = COPY_KIB / cf, COPY_KIB / cw
+        print(f"\n## HBM traffic per launch\n\nThe 1 GiB copy kernel reads FETCH_SIZE = {cf:,.0f} KiB and WRITE_SIZE = {cw:,.0f} KiB "
+              f"for a true 1 048 576 KiB each way: scale factors x {sf:.3f} and x {sw:.3f}.\n")
+        print("| kernel | FETCH_SIZE (KiB) | WRITE_SIZE (KiB) | read, scaled | written, scaled | total |\n|---|---|---|---|---|---|")
+        lines = []
+        for name in sorted(fetch):
+            if not any(k in name for k in OURS) or "FETCH_SIZE" not in fetch[name] or name not in write:
+                continue
+            f_kib, w_kib = fetch[name]["FETCH_SIZE"][0], write[name]["WRITE_SIZE"][0]
+            rd, wr = f_kib * sf * 1024, w_kib * sw * 1024
+            print(f"| {name} | {f_kib:,.0f} | {w_kib:,.0f} | {rd / 1e6:.1f} MB | {wr / 1e6:.1f} MB | {(rd + wr) / 1e6:.1f} MB |")
+            lines.append(f"HBM_TRAFFIC {name} bytes_per_launch={int(rd + wr)} measured_at={commit}")
+        print("\nRead back by bench.py (`roofline.traffic`):\n")
+        for l in lines:
+            print(l)
+
+    for run in ("sq1", "sq2"):
+        path = p(run, "r_counter_collection.csv")
+        if not os.path.exists(path):
+            continue
+        cs = counters(path)
+        names = sorted(k for k in cs if any(o in k for o in ("retention_",)))
+        ctrs = sorted({c for k in names for c in cs[k]})
+        print(f"\n## Shader counters per launch ({run})\n")
+        print("| counter | " + " | ".join(names) + " |\n|---|" + "---|" * len(names))
+        for c in ctrs:
+            print(f"| {c} | " + " | ".join(f"{cs[k][c][0]:,.0f}" if c in cs[k] else "" for k in names) + " |")
+
+
+if __name__ == "__main__":
+    main()

@@ -132,9 +132,12 @@ int fp_pop_retention_bwd(const void* q, const void* k, const void* v, const void
  * [s0, block states] (pop_retnet.py:163-165) does not happen.
  *   q_sfx, k_sfx  [B * (N + 1), sfx_len, H, dk], v_sfx, o_sfx [B * (N + 1), sfx_len, H, dv], block
  *                 index fastest, N = T / block_size, as the reference batches its suffixes
- *   s_out         out: state after the last block, the reference's `last_state` (pop_retnet.py:169);
- *                 may be NULL
- * Needs T % block_size == 0 (as the reference's layer does) and 1 <= sfx_len <= 64. */
+ *   s_out         out: state after the last full block, the reference's `last_state`
+ *                 (pop_retnet.py:169); s0 (zeros if NULL) when T < block_size; may be NULL
+ * T need not be a multiple of block_size: the tokens after the last block boundary are context like
+ * any others (they see the state and each other) and no suffix follows them.  sfx_len >= 1; a suffix
+ * longer than 64 tokens is walked in parts of 64, like a sequence of its own that starts from the
+ * state at its boundary (dk and dv of 64 or 128 only). */
 int fp_pop_fused_fwd(const void* q, const void* k, const void* v, const void* s0, const void* q_sfx, const void* k_sfx,
                      const void* v_sfx, const double* head_decays, void* o, void* o_sfx, void* s_out, int B, int T,
                      int H, int dk, int dv, int block_size, int sfx_len, void* stream);
@@ -182,14 +185,6 @@ int fp_gated_group_norm_fwd(const void* r, const void* g, void* out, long long r
                             void* stream);
 int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, void* d_r, void* d_g, long long rows, int H,
                             int dv, double eps, void* stream);
-
-/* Measurement aid with no counterpart in the reference: streams the tensors of one pass in the
- * pass kernel's access pattern (same grid, same workgroup placement, one chunk of loads in
- * flight) without staging, barriers or arithmetic.  x, w [B,T,H,dA] are read, z [B,T,H,dB] is
- * copied to y.  Its duration is the floor for a pass over these layouts; bench.py reports it
- * beside the pass time.  T a multiple of 64, dA = 128, dB a multiple of 64. */
-int fp_probe_stream_pattern(const void* x, const void* w, const void* z, void* y, int B, int T, int H, int dA, int dB,
-                            void* stream);
 
 /* Message for the last nonzero return on this thread ("" if none). */
 const char* fp_last_error(void);

@@ -109,8 +109,6 @@ FP_DEVICE u32x2 lds_read_tr16_b64(const uint16_t* p) {
   return v;
 }
 
-FP_DEVICE int dbg_flags() { return 0; }
-FP_DEVICE void prof_stamp(int, int) {}
 
 struct BufView {
   const char* base;

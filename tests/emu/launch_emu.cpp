@@ -6,7 +6,6 @@
 #include "retention_bwd_fused.h"
 #include "decode_step.h"
 #include "layer_ops.h"
-#include "stream_probe.h"
 
 #include <thread>
 #include <vector>
@@ -171,22 +170,4 @@ int fpk_launch_gated_norm(const fpk::GatedNormArgs& a, void* /*stream*/, const c
     if (a.out) fpk::gated_norm_fwd(a);
     else fpk::gated_norm_bwd(a);
   });
-}
-
-int fpk_launch_stream_probe(const fpk::StreamProbeArgs& a, void* /*stream*/, const char** err) {
-  long long blocks = 0;
-  if (const char* why = fpk::plan_stream_probe(a, blocks)) {
-    *err = why;
-    return 1;
-  }
-  // no barriers and no lane exchanges inside: the lanes can run one after another on this thread
-  for (long long blk = 0; blk < blocks; ++blk) {
-    for (int t = 0; t < fpk::PROBE_THREADS; ++t) {
-      fprt::g_lane.tid = t;
-      fprt::g_lane.block = (int)blk;
-      fprt::g_lane.grid = (int)blocks;
-      fpk::stream_probe(a, fpk::place_workgroup((int)blk, (int)blocks, 1).wg);
-    }
-  }
-  return 0;
 }

@@ -326,14 +326,6 @@ def oracle_gated_norm_grads(r, g, d_out, eps=1e-6):
     return rf.grad, gf.grad
 
 
-def raw_stream_probe(lib, x, w, z, stream=None):
-    """x, w [B,T,H,dA], z [B,T,H,dB] -> y (a copy of z made in the pass kernel's access pattern)."""
-    B, T, H, dA = x.shape
-    y = torch.full_like(z, float("nan"))
-    _check(lib, lib.fp_probe_stream_pattern(_p(x), _p(w), _p(z), _p(y), B, T, H, dA, z.shape[3], stream))
-    return y
-
-
 def raw_ckpt_fwd_bwd(lib, q, k, v, s, decays, d_o, d_s, every, stream=None):
     """fp_retention_fwd_ckpt followed by fp_retention_bwd_ckpt with checkpoints every `every` tokens.
     Returns (o, S, dq, dk, dv, ds0)."""

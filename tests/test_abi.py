@@ -51,12 +51,12 @@ def test_argument_checks_return_codes(lib):
     bad0 = (ctypes.c_double * 2)(0.0, 0.5)
     assert lib.fp_retention_fwd(p, p, p, null, bad0, p, null, *ok_dims, None) == -4
     assert lib.fp_retention_bwd(p, p, p, null, dec, null, null, p, p, p, null, *ok_dims, None) == -1
-    # fused POP op: T a multiple of the block, suffix length 1..64, head dims of 64, 128 or 256, no NULL tensors
+    # fused POP op: positive block size and suffix length, head dims of 64, 128 or 256, no NULL tensors
     fused = lambda T, dk, blk, ls, o_sfx=p: lib.fp_pop_fused_fwd(p, p, p, null, p, p, p, dec, p, o_sfx, null,
                                                                  1, T, 2, dk, 64, blk, ls, None)
-    assert fused(100, 64, 64, 16) == -2 and b"multiple of block_size" in lib.fp_last_error()
-    assert fused(128, 64, 64, 65) == -2 and b"suffix length" in lib.fp_last_error()
-    assert fused(128, 64, 64, 0) == -2
+    assert fused(100, 64, 0, 16) == -2 and b"block_size" in lib.fp_last_error()
+    assert fused(128, 64, 64, 0) == -2 and b"suffix length" in lib.fp_last_error()
+    assert fused(128, 256, 64, 65) == -3 and b"suffixes longer than" in lib.fp_last_error()
     assert fused(128, 96, 64, 16) == -3
     assert fused(128, 64, 64, 16, null) == -1
     assert lib.fp_pop_fused_bwd(p, p, p, null, p, p, p, dec, p, null, null, p, p, p, p, p, p, null,
@@ -142,15 +142,6 @@ def test_layer_wrappers_refuse_cpu_tensors_and_bad_shapes():
         XPos(128)(q, q, 0)
     with pytest.raises(RuntimeError, match="GPU only"):
         gated_group_norm(q, q.flatten(-2))
-
-
-def test_stream_probe_checks_its_arguments(lib):
-    p, odd, null = ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1008), None
-    assert lib.fp_probe_stream_pattern(p, p, null, p, 1, 64, 2, 128, 64, None) == -1
-    assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 100, 2, 128, 64, None) == -2
-    assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 64, 2, 64, 64, None) == -3
-    assert lib.fp_probe_stream_pattern(p, p, p, p, 1, 64, 2, 128, 96, None) == -3
-    assert lib.fp_probe_stream_pattern(p, odd, p, p, 1, 64, 2, 128, 64, None) == -2
 
 
 def test_pass_ops_refuse_graph_capture(monkeypatch):

@@ -69,17 +69,24 @@ def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
 FUSED_NAMES = ("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0")
 
 
-@pytest.mark.parametrize("B,nblk,block,Ls,H,dk,dv,state_std", [
-    (1, 2, 64, 16, 2, 128, 128, 0.5),    # block == chunk
-    (2, 2, 80, 5, 1, 64, 128, None),     # block of a full and a short chunk, no initial state
-    (1, 3, 24, 64, 1, 128, 64, 0.5),     # block shorter than a chunk, suffix as long as one
-    (1, 1, 130, 1, 1, 64, 64, 0.0),      # one block of three chunks, one-token suffixes
-    (1, 2, 40, 9, 1, 256, 64, 0.5),      # two visits per chunk in the forward and dv passes
-    (1, 2, 64, 16, 1, 64, 256, 0.5),     # ... in the dq and dk passes
+@pytest.mark.parametrize("B,nblk,block,Ls,H,dk,dv,state_std,tail", [
+    (1, 2, 64, 16, 2, 128, 128, 0.5, 0),    # block == chunk
+    (2, 2, 80, 5, 1, 64, 128, None, 0),     # block of a full and a short chunk, no initial state
+    (1, 3, 24, 64, 1, 128, 64, 0.5, 0),     # block shorter than a chunk, suffix as long as one
+    (1, 1, 130, 1, 1, 64, 64, 0.0, 0),      # one block of three chunks, one-token suffixes
+    (1, 2, 40, 9, 1, 256, 64, 0.5, 0),      # two visits per chunk in the forward and dv passes
+    (1, 2, 64, 16, 1, 64, 256, 0.5, 0),     # ... in the dq and dk passes
+    (2, 2, 64, 16, 1, 128, 128, 0.5, 37),   # tokens after the last block boundary (less than a chunk)
+    (1, 1, 150, 7, 2, 64, 128, None, 100),  # ... more than a chunk of them, no initial state
+    (1, 0, 90, 12, 1, 64, 64, 0.5, 70),     # no full block at all: one suffix, read from the initial state
+    (1, 2, 40, 9, 1, 256, 64, 0.5, 11),     # ... with two visits per chunk
+    (1, 2, 64, 100, 1, 128, 128, 0.5, 0),   # suffixes longer than a chunk: two parts
+    (1, 1, 80, 130, 2, 64, 128, None, 30),  # ... three parts, tokens after the last boundary, no initial state
+    (1, 1, 64, 128, 1, 64, 128, 0.3, 0),    # ... two full parts, dk != dv
 ])
-def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std):
+def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std, tail):
     decays = oracle.head_decays(H, (4, 9))
-    T = nblk * block
+    T = nblk * block + tail
     q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + Ls, state_std=state_std)
     sfx = hp.make_suffix_inputs(B, nblk, Ls, H, dk, dv, seed=T + Ls + 1)
     cot = hp.make_cotangents([(B, T, H, dv), tuple(sfx[2].shape), (B, H, dk, dv)], seed=T + 2)
@@ -231,7 +238,3 @@ def test_gated_group_norm(emu_lib, rows, H, dv):
     hp.assert_close(d_g, d_g_ref, "d_g")
 
 
-def test_stream_probe_copies_z(emu_lib):
-    q, k, v, _ = hp.make_inputs(2, 128, 3, 128, 128, seed=12, state_std=None)
-    y = hp.raw_stream_probe(emu_lib, q, k, v)
-    assert torch.equal(y, v)

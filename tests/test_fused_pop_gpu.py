@@ -17,10 +17,12 @@ def _say(msg):
 
 
 def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, oracle_batches=None, d_last=True,
-              oracle_device="cpu", literal=None):
+              oracle_device="cpu", literal=None, tail=0):
+    """N full blocks followed by `tail` < block tokens; N + 1 suffixes of Ls tokens per sequence."""
     from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
-    T = N * block
-    _say(f"[fused pop] B{B} N{N} block{block} Ls{Ls} H{H} dk{dk} dv{dv} s0={state_std} seed={seed}")
+    assert 0 <= tail < block
+    T = N * block + tail
+    _say(f"[fused pop] B{B} N{N} block{block} tail{tail} Ls{Ls} H{H} dk{dk} dv{dv} s0={state_std} seed={seed}")
     decays = oracle.head_decays(H, decay_range)
     q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=seed, state_std=state_std)
     sfx = hp.make_suffix_inputs(B, N, Ls, H, dk, dv, seed=seed + 1)
@@ -69,6 +71,26 @@ def test_fused_parity_sweep(B, N, block, Ls, H, dk, dv):
     run_fused(B, N, block, Ls, H, dk, dv, 0.3, seed=N * block + Ls, decay_range=(5, 12))
 
 
+@pytest.mark.parametrize("B,N,block,Ls,H,dk,dv,tail", [
+    (2, 3, 64, 16, 4, 128, 128, 40),     # tokens after the last block boundary, fewer than a chunk
+    (2, 2, 144, 16, 2, 64, 128, 100),    # ... more than a chunk (the reference's generation block size)
+    (2, 0, 500, 9, 2, 64, 64, 300),      # no full block: one suffix per sequence, reading the initial state
+    (1, 2, 64, 16, 2, 256, 128, 17),     # with two visits per chunk
+    (2, 3, 64, 100, 4, 128, 128, 0),     # suffixes longer than a chunk: two parts
+    (1, 2, 96, 200, 2, 64, 128, 50),     # four parts and a tail
+    (1, 2, 64, 128, 2, 128, 64, 0),      # two full parts, dk != dv
+])
+def test_fused_trailing_tokens_and_long_suffixes(B, N, block, Ls, H, dk, dv, tail):
+    """What the reference's layer accepts beyond whole blocks and short suffixes: T % block_size != 0
+    (the context goes on after the last boundary, last_state stays the last full block's,
+    flash_pop/pop_retnet.py:169) and suffixes of any length."""
+    run_fused(B, N, block, Ls, H, dk, dv, 0.3, seed=N * block + Ls + tail, decay_range=(5, 12), tail=tail)
+    # (without a full block and without an initial state the reference's layer has no state batch to
+    # build its suffix call from, pop_retnet.py:161-164, and the oracle follows it: zeros instead)
+    run_fused(B, N, block, Ls, H, dk, dv, None if N else 0.0, seed=N * block + Ls + tail + 1, decay_range=(5, 12), tail=tail,
+              d_last=False)
+
+
 def test_fused_without_state_and_without_last_state_gradient():
     run_fused(2, 3, 64, 8, 2, 64, 64, None, seed=5)
     run_fused(1, 2, 96, 8, 2, 128, 128, 0.2, seed=6, d_last=False)
@@ -115,13 +137,8 @@ def test_fused_argument_errors():
     decays = oracle.head_decays(2)
     q, k, v, s = hp.make_inputs(1, 128, 2, 64, 64, seed=1, state_std=0.1, device=DEV)
     sfx = hp.make_suffix_inputs(1, 2, 8, 2, 64, 64, seed=2, device=DEV)
-    with pytest.raises(ValueError, match="multiple of block_size"):
-        flash_pop_retention_with_suffixes(q, k, v, s, decays, 50, *sfx)
     with pytest.raises(ValueError, match="one additional suffix block"):
         flash_pop_retention_with_suffixes(q, k, v, s, decays, 32, *sfx)
-    long_sfx = hp.make_suffix_inputs(1, 2, 65, 2, 64, 64, seed=3, device=DEV)
-    with pytest.raises(RuntimeError, match="suffix length"):
-        flash_pop_retention_with_suffixes(q, k, v, s, decays, 64, *long_sfx)
 
 
 def test_config4_fused():
