@@ -197,13 +197,31 @@ int checkpoint_interval(const Shape& s) {
   return every;
 }
 
+// Suffix tensors of one fused POP call, in the roles q, k, v / d_o (inputs) and o / dq, dk, dv (outputs)
+struct Suffixes {
+  const void *q, *k, *v;
+  int len;
+};
+struct SuffixGrads {
+  const void* d_o;
+  void *dq, *dk, *dv;
+  int block;
+};
+
 int backward_fused(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
                    const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, void* stream,
-                   const void* ckpt = nullptr, int ckpt_every = 0) {
+                   const void* ckpt = nullptr, int ckpt_every = 0, const Suffixes* sfx = nullptr,
+                   const SuffixGrads* sg = nullptr) {
   fpk::FusedBwdArgs a;
   std::memset(&a, 0, sizeof a);
   a.ckpt = in(ckpt);
   a.ckpt_every = ckpt ? ckpt_every : 0;
+  if (sfx) {
+    a.q_sfx = in(sfx->q); a.k_sfx = in(sfx->k); a.v_sfx = in(sfx->v); a.dO_sfx = in(sg->d_o);
+    a.dq_sfx = out(sg->dq); a.dk_sfx = out(sg->dk); a.dv_sfx = out(sg->dv);
+    a.block = sg->block;
+    a.Ls = sfx->len;
+  }
   a.q = in(q); a.k = in(k); a.v = in(v); a.dO = in(d_o);
   a.dq = out(dq); a.dk = out(dk_); a.dv = out(dv_);
   a.s0 = in(s0); a.ds_out = in(d_s_out); a.ds0 = out(d_s0);
@@ -384,12 +402,6 @@ int check_workspace(const Shape& s, int segments, const void* workspace, size_t 
   return FP_OK;
 }
 
-// Suffix tensors of one fused POP call, in the roles q, k, v / d_o (inputs) and o / dq, dk, dv (outputs)
-struct Suffixes {
-  const void *q, *k, *v;
-  int len;
-};
-
 int check_fused(const Shape& s, int block, int sfx_len) {
   if (block < 1) return fail(FP_ERR_BAD_SHAPE, "block_size must be >= 1 (got %d)", block);
   if (sfx_len < 1) return fail(FP_ERR_BAD_SHAPE, "suffix length must be positive (got %d)", sfx_len);
@@ -425,6 +437,11 @@ int fused_forward(const Shape& s, const void* q, const void* k, const void* v, c
 int fused_backward(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const Suffixes& x,
                    const double* decays, const void* d_o, const void* d_o_sfx, const void* d_s_out, void* dq, void* dk_,
                    void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx, void* d_s0, int block, void* stream) {
+  // whole 64-token chunks per block, suffixes of one chunk at most: the kernel that carries dS once
+  if (use_fused_backward(s, nullptr) && block % fpk::CH == 0 && s.T % block == 0 && x.len <= fpk::CH) {
+    const SuffixGrads sg{d_o_sfx, dq_sfx, dk_sfx, dv_sfx, block};
+    return backward_fused(s, q, k, v, s0, decays, d_o, d_s_out, dq, dk_, dv_, d_s0, stream, nullptr, 0, &x, &sg);
+  }
   const float sc = 1.0f / std::sqrt((float)s.dk);
   fpk::PassArgs g, a;
 

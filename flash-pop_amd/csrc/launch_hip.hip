@@ -33,7 +33,13 @@ __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_multi_kernel(
 
 __global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_kernel(const fpk::FusedBwdArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::fused_bwd(args, lds, fprt::block_index());
+  fpk::fused_bwd<false>(args, lds, fprt::block_index());
+}
+
+// the same with POP suffixes at the block boundaries
+__global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_pop_kernel(const fpk::FusedBwdArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::fused_bwd<true>(args, lds, fprt::block_index());
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -62,7 +68,7 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(cons
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
-static_assert(2 * fpk::PASS_KERNELS <= 62, "one bit per kernel instantiation, single and paired");
+static_assert(2 * fpk::PASS_KERNELS <= 61, "one bit per kernel instantiation, single and paired");
 std::atomic<uint64_t> g_armed[kMaxDevices];
 
 template <typename Kernel, typename... More>
@@ -192,9 +198,8 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
 }
 
 int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* stream, const char** err) {
-  if (a.B < 1 || a.T < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || (long long)a.B * a.H * 2 > 0x7fffffffLL || !a.q || !a.k ||
-      !a.v || !a.dO || !a.dq || !a.dk || !a.dv) {
-    *err = "fused backward: bad arguments";
+  if (const char* why = fpk::check_fused_bwd(a)) {
+    *err = why;
     return 1;
   }
   int dev = 0;
@@ -202,19 +207,25 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* stream, const char** 
     *err = "hipGetDevice failed";
     return 1;
   }
-  // the opt-in to more than 64 KB of LDS, once per device (the top bit of the per-device word)
+  const bool pop = a.block > 0;
+  const void* const kernel = pop ? reinterpret_cast<const void*>(retention_bwd_fused_pop_kernel)
+                                 : reinterpret_cast<const void*>(retention_bwd_fused_kernel);
+  // the opt-in to more than 64 KB of LDS, once per device (the top bits of the per-device word)
+  const uint64_t bit = 1ull << (pop ? 62 : 63);
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1ull << 63))) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(retention_bwd_fused_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, fpk::fb_lds_bytes()) != hipSuccess) {
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & bit)) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, fpk::fb_lds_bytes()) != hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(1ull << 63, std::memory_order_release);
+    if (tracked) g_armed[dev].fetch_or(bit, std::memory_order_release);
   }
-  hipLaunchKernelGGL(retention_bwd_fused_kernel, dim3((unsigned)(2 * a.B * a.H)), dim3(fpk::FB_THREADS), fpk::fb_lds_bytes(),
-                     static_cast<hipStream_t>(stream), a);
+  const dim3 grid((unsigned)(2 * a.B * a.H)), threads(fpk::FB_THREADS);
+  if (pop)
+    hipLaunchKernelGGL(retention_bwd_fused_pop_kernel, grid, threads, fpk::fb_lds_bytes(), static_cast<hipStream_t>(stream), a);
+  else
+    hipLaunchKernelGGL(retention_bwd_fused_kernel, grid, threads, fpk::fb_lds_bytes(), static_cast<hipStream_t>(stream), a);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     *err = hipGetErrorString(e);

@@ -122,6 +122,12 @@ struct FusedBwdArgs {
   // the other finds in the caches.  Null: one forward walk from s0.
   const uint16_t* ckpt;
   int ckpt_every;
+  // POP suffixes (block > 0; none of the above checkpoints then): one suffix of Ls <= 64 tokens per
+  // block boundary 0, block, ..., T, tensors [B * (T / block + 1), Ls, H, 128] as in PassArgs; block a
+  // multiple of 64 that divides T.  A suffix reads the state at its boundary without advancing it.
+  const uint16_t *q_sfx, *k_sfx, *v_sfx, *dO_sfx;
+  uint16_t *dq_sfx, *dk_sfx, *dv_sfx;
+  int block, Ls;
   int B, T, H;
   float scale;                             // dk^-1/2
   float log2g[MAX_HEADS];

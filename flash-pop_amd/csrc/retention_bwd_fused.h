@@ -107,7 +107,42 @@ struct Common {
   uint32_t rowp;          // bytes between consecutive tokens of a tensor
   float lg;
   int ld_row, ld_piece;   // this thread's 16-byte pieces of a tile: rows ld_row and ld_row + 32
+  // POP suffixes (SFX instantiations): block = tokens per block (a multiple of CH that divides T),
+  // Ls <= CH tokens per suffix, nblk = T / block, spb = chunks per block
+  int block, Ls, nblk, spb;
 };
+
+// One stop of a walk: a chunk of the sequence or, with POP suffixes, the suffix that hangs off a
+// block boundary.  `row` is its first row among all rows of its tensors ([B * T] rows; suffixes:
+// [B * (nblk + 1) * Ls] rows); L = 0 stands for "beyond the walk".
+struct Item {
+  uint32_t row;
+  int L;
+  bool sfx;
+};
+FP_DEVICE Item chunk_item(const Common& k, int ci) {
+  if (ci < 0 || ci >= k.nch) return Item{0u, 0, false};
+  const int t0 = ci * CH;
+  return Item{(uint32_t)k.b * k.T + t0, k.T - t0 < CH ? k.T - t0 : CH, false};
+}
+FP_DEVICE Item suffix_item(const Common& k, int n) { return Item{((uint32_t)k.b * (k.nblk + 1) + n) * k.Ls, k.Ls, true}; }
+// Walking backward with suffixes: the suffix at T, then per block (from the last) its chunks
+// from the last to the first and the suffix at its lower boundary.
+FP_DEVICE Item item_backward(const Common& k, int it) {
+  if (k.block == 0) return chunk_item(k, k.nch - 1 - it);
+  if (it <= 0) return it == 0 ? suffix_item(k, k.nblk) : Item{0u, 0, false};
+  const int j = it - 1, blk = k.nblk - 1 - j / (k.spb + 1), r = j % (k.spb + 1);
+  if (blk < 0) return Item{0u, 0, false};
+  return r < k.spb ? chunk_item(k, (blk + 1) * k.spb - 1 - r) : suffix_item(k, blk);
+}
+// Walking forward with suffixes: per block the suffix at its lower boundary and its chunks, then the suffix at T.
+FP_DEVICE Item item_forward(const Common& k, int it) {
+  if (k.block == 0) return chunk_item(k, it);
+  const int blk = it / (k.spb + 1), r = it % (k.spb + 1);
+  if (it < 0 || blk > k.nblk || (blk == k.nblk && r > 0)) return Item{0u, 0, false};
+  return r == 0 ? suffix_item(k, blk) : chunk_item(k, blk * k.spb + r - 1);
+}
+FP_DEVICE int item_count(const Common& k) { return k.block == 0 ? k.nch : 1 + k.nblk * (k.spb + 1); }
 
 FP_DEVICE Common make_common(const FusedBwdArgs& p, int stream) {
   Common k;
@@ -124,24 +159,31 @@ FP_DEVICE Common make_common(const FusedBwdArgs& p, int stream) {
   k.lg = p.log2g[k.h];
   k.ld_row = k.tid >> 4;
   k.ld_piece = k.tid & 15;
+  k.block = p.block;
+  k.Ls = p.Ls;
+  k.nblk = p.block > 0 ? p.T / p.block : 0;
+  k.spb = p.block / CH;
   return k;
 }
 
-// view of the rows of chunk `ci` of one tensor for this stream; rows past the sequence read as
-// zero and are dropped on stores
-FP_DEVICE fprt::BufView chunk_view(const Common& k, const void* base, int ci, bool store = false) {
-  const bool ok = ci >= 0 && ci < k.nch;
-  const int t0 = ok ? ci * CH : 0;
-  const int L = ok ? (k.T - t0 < CH ? k.T - t0 : CH) : 0;
-  const char* ptr = static_cast<const char*>(base) + ((size_t)k.b * k.T + t0) * k.rowp + (size_t)k.h * FB_D * 2;
-  return fprt::make_buf(ptr, L > 0 ? (uint32_t)(L - 1) * k.rowp + FB_D * 2 : 0u);
+// view of the rows of an item in one tensor (`ctx` for chunks, `sfx` for suffixes) for this
+// stream; rows past the item read as zero and are dropped on stores
+FP_DEVICE fprt::BufView item_view(const Common& k, const void* ctx, const void* sfx, const Item& it) {
+  const char* ptr = static_cast<const char*>(it.sfx ? sfx : ctx) + (size_t)it.row * k.rowp + (size_t)k.h * FB_D * 2;
+  return fprt::make_buf(ptr, it.L > 0 ? (uint32_t)(it.L - 1) * k.rowp + FB_D * 2 : 0u);
 }
 
+// the tensors of a role in the chunk tensors and in the suffix tensors
 template <int N>
-FP_DEVICE void load_tiles(const Common& k, const void* const (&src)[N], int ci, u32x4 (&pf)[2 * N]) {
+struct Sources {
+  const void* ctx[N];
+  const void* sfx[N];
+};
+template <int N>
+FP_DEVICE void load_tiles(const Common& k, const Sources<N>& src, const Item& it, u32x4 (&pf)[2 * N]) {
 #pragma unroll
   for (int x = 0; x < N; ++x) {
-    const fprt::BufView v = chunk_view(k, src[x], ci);
+    const fprt::BufView v = item_view(k, src.ctx[x], src.sfx[x], it);
 #pragma unroll
     for (int u = 0; u < 2; ++u)
       pf[2 * x + u] = fprt::buf_load128(v, (uint32_t)(k.ld_row + 32 * u) * k.rowp + k.ld_piece * 16);
@@ -158,9 +200,9 @@ FP_DEVICE void stage_tiles(const Common& k, uint16_t* tiles, const u32x4 (&pf)[2
     }
   }
 }
-// staging tile ([token][feature]) -> rows of chunk ci of `dst`
-FP_DEVICE void drain_tile(const Common& k, const uint16_t* tile, void* dst, int ci) {
-  const fprt::BufView v = chunk_view(k, dst, ci, true);
+// staging tile ([token][feature]) -> rows of an item in `dst` (chunks) or `dst_sfx` (suffixes)
+FP_DEVICE void drain_tile(const Common& k, const uint16_t* tile, void* dst, void* dst_sfx, const Item& it) {
+  const fprt::BufView v = item_view(k, dst, dst_sfx, it);
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int row = k.ld_row + 32 * u;
@@ -297,7 +339,11 @@ FP_DEVICE void score_weights(float s_intra, float lg, bool diagonal, bool revers
 //      tiles of the next chunk replace the ones nobody reads any more; the new copy of dS
 //   3  the q and dO tiles of the next chunk
 // The outputs leave for global memory at the start of the next chunk's first stretch.
-template <int PASS>
+//
+// SFX: POP suffixes hang off the block boundaries (item_backward).  Nothing downstream of a suffix
+// reaches back into it, so it reads no dS (no read-out), and what it adds to dS, the gradient of
+// the state it read, is not decayed.
+template <int PASS, bool SFX>
 FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   using namespace fb;
   const Common k = make_common(p, stream);
@@ -336,16 +382,18 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   const float wread_full1 = p.scale * fprt::exp2_approx((float)(CH - 1 - 32 - c) * lg);
   const float gL_full = fprt::exp2_approx((float)CH * lg);
 
-  const void* const src_qg[2] = {p.q, p.dO};
-  const void* const src_kv[2] = {p.k, p.v};
+  const Sources<2> src_qg = {{p.q, p.dO}, {p.q_sfx, p.dO_sfx}};
+  const Sources<2> src_kv = {{p.k, p.v}, {p.k_sfx, p.v_sfx}};
+  const int nitems = item_count(k);
+  Item cur = item_backward(k, 0), nxt = item_backward(k, 1), prev = cur;
   u32x4 pf_qg[4], pf_kv[4];
-  load_tiles<2>(k, src_qg, k.nch - 1, pf_qg);
-  load_tiles<2>(k, src_kv, k.nch - 1, pf_kv);
+  load_tiles<2>(k, src_qg, cur, pf_qg);
+  load_tiles<2>(k, src_kv, cur, pf_kv);
   load_state(k, Rt, p.ds_out ? p.ds_out + (size_t)stream * FB_D * FB_D : nullptr, false);
   stage_tiles<2>(k, TL, pf_qg);
   stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
-  load_tiles<2>(k, src_qg, k.nch - 2, pf_qg);
-  load_tiles<2>(k, src_kv, k.nch - 2, pf_kv);
+  load_tiles<2>(k, src_qg, nxt, pf_qg);
+  load_tiles<2>(k, src_kv, nxt, pf_kv);
   fprt::block_sync();
   f32x16 racc[2];
 #pragma unroll
@@ -355,12 +403,14 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   const uint16_t* const xrow1 = Xs + at(32 + c, 8 * g);
   const uint16_t* const rrow = Rt + at(32 * rt + c, 8 * g);
 
-  for (int ci = k.nch - 1; ci >= 0; --ci) {
-    const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
-    // ---- the previous chunk's outputs leave (nothing writes the staging tiles before the next barrier)
-    if (ci < k.nch - 1) {
-      drain_tile(k, OUT, p.dv, ci + 1);
-      drain_tile(k, OUT + FB_TILE, p.dk, ci + 1);
+  for (int it = 0; it < nitems; ++it) {
+    const int L = cur.L;
+    const bool sfx = SFX && cur.sfx;
+    const Item after = item_backward(k, it + 2);
+    // ---- the previous item's outputs leave (nothing writes the staging tiles before the next barrier)
+    if (it > 0) {
+      drain_tile(k, OUT, p.dv, p.dv_sfx, prev);
+      drain_tile(k, OUT + FB_TILE, p.dk, p.dk_sfx, prev);
     }
     // ---- stretch 1: scores D[j][i] = W[j] . X[i] and read-out wread(i) sum_a R^T[n][a] X[i][a], the
     // operands of a k-step requested a few k-steps ahead
@@ -377,7 +427,19 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
         ra[t] = pass == 0 ? frag_cols(rrow, t) : frag_rows(Rt, tr_seq, t, 32 * rt);
       };
       constexpr int AHEAD = 3;   // k-steps of operands in flight
-      if (scores) {
+      if (sfx) {   // no read-out: only the score tile
+        if (scores) {
+#pragma unroll
+          for (int t = 0; t < 8; ++t) {
+            wf[t] = frag_cols(s_wrow, t);
+            x0[t] = frag_cols(s_ib ? xrow1 : xrow0, t);
+          }
+          fprt::sched_fence();
+#pragma unroll
+          for (int t = 0; t < 8; ++t) sc = fprt::mfma_32x32x16_bf16(wf[t], x0[t], sc);
+          score_finish(sc, mw, s_jb == s_ib, true, c, g, xp_pass + rt * FB_XP, lane);
+        }
+      } else if (scores) {
 #pragma unroll
         for (int t = 0; t < AHEAD; ++t) request(t);
         fprt::sched_fence();
@@ -445,7 +507,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       fprt::sched_fence();
       put_output(out, c, 32 * rt, g, acc[0]);
       put_output(out, 32 + c, 32 * rt, g, acc[1]);
-      const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
+      const float gL = sfx ? 1.f : L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
 #pragma unroll
@@ -470,18 +532,21 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     }
     // nobody reads this chunk's k and v tiles or the old copy of dS any more
     stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
-    load_tiles<2>(k, src_kv, ci - 2, pf_kv);
+    load_tiles<2>(k, src_kv, after, pf_kv);
 #pragma unroll
     for (int u = 0; u < 2; ++u) put_state(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
     fprt::block_sync();
 
     // ---- stretch 3: every read of this chunk's q and dO tiles is done
     stage_tiles<2>(k, TL, pf_qg);
-    load_tiles<2>(k, src_qg, ci - 2, pf_qg);
+    load_tiles<2>(k, src_qg, after, pf_qg);
     fprt::block_sync();
+    prev = cur;
+    cur = nxt;
+    nxt = after;
   }
-  drain_tile(k, OUT, p.dv, 0);
-  drain_tile(k, OUT + FB_TILE, p.dk, 0);
+  drain_tile(k, OUT, p.dv, p.dv_sfx, prev);
+  drain_tile(k, OUT + FB_TILE, p.dk, p.dk_sfx, prev);
   if (p.ds0) store_state(k, Rt, p.ds0 + (size_t)stream * FB_D * FB_D, false);
 }
 
@@ -490,7 +555,9 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
 // Waves 0..3 ("output") own rows 32 w .. of Y^T = dq^T for both 32-token halves; waves 4..7
 // ("state") make the score tiles and own the four tiles of rows 32 (w - 4) .. of R.
 // STATE: the copy that waves 4..7 run; the two copies meet at the same barriers.
-template <bool STATE>
+// SFX: POP suffixes hang off the block boundaries (item_forward): a suffix reads R without
+// advancing it (no checkpoints in this form).
+template <bool STATE, bool SFX>
 FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
   using namespace fb;
   const Common k = make_common(p, stream);
@@ -531,17 +598,21 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     const size_t nck = (size_t)(k.T / p.ckpt_every);
     return p.ckpt + (((size_t)k.b * nck + (seg - 1)) * p.H + k.h) * FB_D * FB_D;
   };
-  const void* const src_x[1] = {p.dO};
-  const void* const src_wz[2] = {p.v, p.k};
+  // item visited in iteration `it`
+  auto item_of = [&](int it) { return SFX ? item_forward(k, it) : chunk_item(k, chunk_of(it)); };
+  const int nitems = SFX ? item_count(k) : k.nch;
+  const Sources<1> src_x = {{p.dO}, {p.dO_sfx}};
+  const Sources<2> src_wz = {{p.v, p.k}, {p.v_sfx, p.k_sfx}};
+  Item cur = item_of(0), nxt = item_of(1), prev = cur;
   u32x4 pf_x[2], pf_wz[4];
-  load_tiles<1>(k, src_x, chunk_of(0), pf_x);
-  load_tiles<2>(k, src_wz, chunk_of(0), pf_wz);
+  load_tiles<1>(k, src_x, cur, pf_x);
+  load_tiles<2>(k, src_wz, cur, pf_wz);
   // R[a][n] = S[n][a]: element (a, n) at n * 128 + a of a state matrix
   load_state(k, Rt, segment_state(nseg - 1), true);
   stage_tiles<1>(k, TL, pf_x);
   stage_tiles<2>(k, TL + FB_TILE, pf_wz);
-  load_tiles<1>(k, src_x, chunk_of(1), pf_x);
-  load_tiles<2>(k, src_wz, chunk_of(1), pf_wz);
+  load_tiles<1>(k, src_x, nxt, pf_x);
+  load_tiles<2>(k, src_wz, nxt, pf_wz);
   fprt::block_sync();
   f32x16 racc[4];
   if constexpr (state_role) {
@@ -563,11 +634,13 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
   //   2  Y^T += Z^T P^T and the outputs (output waves); the state update and the new copy of R
   //      (state waves); the next chunk's X tile
   //   3  the next chunk's W and Z tiles
-  for (int it = 0; it < k.nch; ++it) {
-    const int ci = chunk_of(it), next = chunk_of(it + 1);
-    const bool fresh = next >= 0 && next != ci + 1;   // the next chunk starts another segment
-    const int L = k.T - ci * CH < CH ? k.T - ci * CH : CH;
-    if (it > 0) drain_tile(k, OUT, p.dq, chunk_of(it - 1));   // nothing writes the staging tile before the next barrier
+  for (int it = 0; it < nitems; ++it) {
+    const int next = SFX ? 0 : chunk_of(it + 1);
+    const bool fresh = !SFX && next >= 0 && next != chunk_of(it) + 1;   // the next chunk starts another segment
+    const bool sfx = SFX && cur.sfx;
+    const int L = cur.L;
+    const Item after = item_of(it + 2);
+    if (it > 0) drain_tile(k, OUT, p.dq, p.dq_sfx, prev);   // nothing writes the staging tile before the next barrier
     f32x16 acc[2];
     if constexpr (state_role) {
       if (rt < 3) {
@@ -630,7 +703,7 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
       }
       put_output(OUT, c, 32 * rt, g, acc[0]);
       put_output(OUT, 32 + c, 32 * rt, g, acc[1]);
-    } else {
+    } else if (!sfx) {
       // R[a][n] = gamma^L R + sum_j s gamma^(L-1-j) W[j][a] Z[j][n]
       const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);
 #pragma unroll
@@ -680,12 +753,12 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     }
     // nobody reads this chunk's X tile or the old copy of R any more
     stage_tiles<1>(k, TL, pf_x);
-    load_tiles<1>(k, src_x, chunk_of(it + 2), pf_x);
+    load_tiles<1>(k, src_x, after, pf_x);
     if (fresh) load_state(k, Rt, segment_state(next / seg_chunks), true);   // the next segment's starting state
     fprt::block_sync();
 
     stage_tiles<2>(k, TL + FB_TILE, pf_wz);
-    load_tiles<2>(k, src_wz, chunk_of(it + 2), pf_wz);
+    load_tiles<2>(k, src_wz, after, pf_wz);
     if constexpr (state_role) {
       if (fresh) {
 #pragma unroll
@@ -693,19 +766,41 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
       }
     }
     fprt::block_sync();
+    prev = cur;
+    cur = nxt;
+    nxt = after;
   }
-  drain_tile(k, OUT, p.dq, chunk_of(k.nch - 1));
+  drain_tile(k, OUT, p.dq, p.dq_sfx, prev);
 }
 
 // launch index -> kind and stream: the reverse workgroups (the longer ones) come first
+// SFX: the form with POP suffixes (p.block > 0)
+template <bool SFX>
 FP_DEVICE void fused_bwd(const FusedBwdArgs& p, char* lds, int block) {
   const int streams = p.B * p.H;
   if (block < streams) {
-    if (fprt::thread_index() < 256) fused_bwd_reverse<0>(p, lds, block);
-    else fused_bwd_reverse<1>(p, lds, block);
+    if (fprt::thread_index() < 256) fused_bwd_reverse<0, SFX>(p, lds, block);
+    else fused_bwd_reverse<1, SFX>(p, lds, block);
   }
-  else if (fprt::thread_index() < 256) fused_bwd_forward<false>(p, lds, block - streams);
-  else fused_bwd_forward<true>(p, lds, block - streams);
+  else if (fprt::thread_index() < 256) fused_bwd_forward<false, SFX>(p, lds, block - streams);
+  else fused_bwd_forward<true, SFX>(p, lds, block - streams);
+}
+
+// What the kernel assumes about its arguments; nullptr or a message for the caller.
+inline const char* check_fused_bwd(const FusedBwdArgs& a) {
+  if (a.B < 1 || a.T < 1 || a.H < 1 || a.H > MAX_HEADS || (long long)a.B * a.H * 2 > 0x7fffffffLL || !a.q || !a.k || !a.v ||
+      !a.dO || !a.dq || !a.dk || !a.dv)
+    return "fused backward: bad arguments";
+  if (a.ckpt && (a.ckpt_every <= 0 || a.ckpt_every % CH != 0 || a.block > 0))
+    return "fused backward: checkpoints every positive multiple of 64 tokens, and not together with suffixes";
+  if (a.block > 0) {
+    if (a.block % CH != 0 || a.T % a.block != 0 || a.Ls < 1 || a.Ls > CH)
+      return "fused backward with suffixes: block a multiple of 64 that divides T, 1 <= Ls <= 64";
+    if (!a.q_sfx || !a.k_sfx || !a.v_sfx || !a.dO_sfx || !a.dq_sfx || !a.dk_sfx || !a.dv_sfx)
+      return "fused backward with suffixes: all seven suffix tensors are needed";
+    if ((long long)a.B * (a.T / a.block + 1) * a.Ls >= (1LL << 32)) return "fused backward with suffixes: too many suffix rows";
+  }
+  return nullptr;
 }
 
 }  // namespace fpk

@@ -107,11 +107,14 @@ int fpk_static_scratch(void** ptr, const char** /*err*/) {
 int fpk_compute_units() { return 8; }
 
 int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* /*stream*/, const char** err) {
-  if (a.B < 1 || a.T < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || !a.q || !a.k || !a.v || !a.dO || !a.dq || !a.dk || !a.dv) {
-    *err = "fused backward: bad arguments";
+  if (const char* why = fpk::check_fused_bwd(a)) {
+    *err = why;
     return 1;
   }
-  return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(), [&](char* l) { fpk::fused_bwd(a, l, fprt::block_index()); });
+  return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(), [&](char* l) {
+    if (a.block > 0) fpk::fused_bwd<true>(a, l, fprt::block_index());
+    else fpk::fused_bwd<false>(a, l, fprt::block_index());
+  });
 }
 
 int fpk_launch_scan(const fpk::ScanArgs& a, void* /*stream*/, const char** err) {

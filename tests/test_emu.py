@@ -114,6 +114,31 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
 
 
+@pytest.mark.parametrize("B,nblk,block,Ls,H,state_std", [
+    (1, 4, 128, 16, 2, 0.5),     # two chunks per block
+    (2, 8, 64, 64, 1, None),     # block == chunk, suffixes as long as a chunk, no initial state
+    (1, 3, 192, 1, 2, 0.3),      # three chunks per block, one-token suffixes
+])
+def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, block, Ls, H, state_std):
+    """dk = dv = 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
+    the kernel that walks backward once for dk and dv beside a forward walk for dq, with the
+    suffixes as extra stops at the block boundaries.  Same results as the pass-per-gradient path."""
+    decays = oracle.head_decays(H, (4, 9))
+    T = nblk * block
+    q, k, v, s = hp.make_inputs(B, T, H, 128, 128, seed=T + Ls, state_std=state_std)
+    sfx = hp.make_suffix_inputs(B, nblk, Ls, H, 128, 128, seed=T + Ls + 1)
+    cot = hp.make_cotangents([(B, T, H, 128), tuple(sfx[2].shape), (B, H, 128, 128)], seed=T + 2)
+    monkeypatch.setenv("FLASHPOP_BWD", "fused")
+    grads = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
+    _, _, _, g_ref = hp.oracle_fused(q, k, v, s, sfx, decays, block, cot)
+    _check_all([(n, g, r) for n, g, r in zip(FUSED_NAMES, grads, g_ref)])
+    monkeypatch.setenv("FLASHPOP_BWD", "passes")
+    other = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
+    for name, x, y in zip(FUSED_NAMES, grads, other):
+        if x is not None:
+            assert hp.error_report(x, y.float())["rms_ratio"] < 0.004, name
+
+
 @pytest.mark.parametrize("B,T,H,state_std,every", [
     (1, 700, 2, 0.5, 128),      # ragged tail beyond the last checkpoint, initial state
     (1, 512, 1, None, 256),     # the sequence ends on a checkpoint, no initial state
