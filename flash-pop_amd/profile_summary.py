@@ -52,6 +52,46 @@ def copy_reading(path, counter):
     return best
 
 
+FAMILIES = (
+    ("retention kernels of this library", ("retention_", "segment_scan", "decode_step")),
+    ("rotary embedding kernel of this library", ("rotary_qk",)),
+    ("norm + gate kernels of this library", ("gated_norm",)),
+    ("GEMMs (rocBLAS / hipBLASLt)", ("Cijk_", "gemm", "Gemm")),
+)
+
+
+def model_breakdown(path):
+    """Where the time of the traced run goes, by kernel family (the run holds bench.py's headline
+    leg and its model leg; the headline leg's 12 forward + backward launches are a fraction of a
+    per cent of it)."""
+    rows = []
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            rows.append((r["Name"], int(r["Calls"]), int(r["TotalDurationNs"])))
+    total = sum(r[2] for r in rows)
+    print("\n## Model-level run (config 5 harness): GPU time by kernel family\n")
+    print("| family | launches | total | share of GPU time |\n|---|---|---|---|")
+    rest_calls, rest_ns = 0, 0
+    fam = {name: [0, 0] for name, _ in FAMILIES}
+    for name, calls, ns in rows:
+        for fname, keys in FAMILIES:
+            if any(k in name for k in keys):
+                fam[fname][0] += calls
+                fam[fname][1] += ns
+                break
+        else:
+            rest_calls += calls
+            rest_ns += ns
+    for fname, _ in FAMILIES:
+        print(f"| {fname} | {fam[fname][0]} | {fam[fname][1] / 1e6:.2f} ms | {100 * fam[fname][1] / total:.1f} % |")
+    print(f"| everything else (torch elementwise, reductions, copies, losses) | {rest_calls} | {rest_ns / 1e6:.2f} ms | {100 * rest_ns / total:.1f} % |")
+    print(f"| all kernels | {sum(r[1] for r in rows)} | {total / 1e6:.2f} ms | 100 % |")
+    print("\nLibrary kernels in this run:\n\n| kernel | calls | average | total |\n|---|---|---|---|")
+    for name, calls, ns in sorted(rows, key=lambda r: -r[2]):
+        if any(k in name for k in OURS):
+            print(f"| {short(name)} | {calls} | {ns / calls / 1e3:.1f} us | {ns / 1e6:.2f} ms |")
+
+
 def main():
     out = sys.argv[1]
     commit = sys.argv[2] if len(sys.argv) > 2 else subprocess.run(
@@ -82,6 +122,9 @@ def main():
         print("\nRead back by bench.py (`roofline.traffic`):\n")
         for l in lines:
             print(l)
+
+    if os.path.exists(p("model_trace", "r_kernel_stats.csv")):
+        model_breakdown(p("model_trace", "r_kernel_stats.csv"))
 
     for run in ("sq1", "sq2"):
         path = p(run, "r_counter_collection.csv")

@@ -62,9 +62,22 @@ int pop(int B, int T, int H, int dk, int dv, int block) {
   return done(rc, "pop", B, T, H, dk, dv, block);
 }
 
-int fused(int B, int nblk, int block, int ls, int H, int dk, int dv) {
+// forward with checkpoints every `every` tokens, then the backward that starts from them
+int checkpointed(int B, int T, int H, int every) {
   std::vector<double> dec(H, 0.97);
-  const int T = nblk * block;
+  const int d = 128;
+  const size_t n = (size_t)B * T * H * d, ns = (size_t)B * H * d * d, nc = (size_t)B * (T / every) * H * d * d;
+  uint16_t *q = buf(n), *k = buf(n), *v = buf(n), *s = buf(ns), *o = buf(n, false), *so = buf(ns, false), *ck = buf(nc, false);
+  uint16_t *dO = buf(n), *dS = buf(ns), *dq = buf(n, false), *dk_ = buf(n, false), *dv_ = buf(n, false), *ds0 = buf(ns, false);
+  int rc = fp_retention_fwd_ckpt(q, k, v, s, dec.data(), o, so, ck, every, B, T, H, d, d, nullptr);
+  if (!rc) rc = fp_retention_bwd_ckpt(q, k, v, s, dec.data(), dO, dS, ck, every, dq, dk_, dv_, ds0, B, T, H, d, d, nullptr);
+  return done(rc, "checkpointed", B, T, H, d, d, every);
+}
+
+// nblk full blocks and `tail` < block tokens after them
+int fused(int B, int nblk, int block, int ls, int H, int dk, int dv, int tail = 0) {
+  std::vector<double> dec(H, 0.97);
+  const int T = nblk * block + tail;
   const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
   const size_t sq = (size_t)B * (nblk + 1) * ls * H * dk, sv = (size_t)B * (nblk + 1) * ls * H * dv;
   uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = buf(ns), *qs = buf(sq), *ks = buf(sq), *vs = buf(sv);
@@ -124,6 +137,12 @@ int main() {
   rc |= fused(2, 2, 80, 5, 1, 64, 128);
   rc |= fused(1, 3, 24, 64, 1, 128, 64);
   rc |= fused(1, 2, 40, 9, 1, 64, 256);       // suffixes with two visits per chunk
+  rc |= fused(1, 1, 80, 5, 1, 64, 128, 30);   // tokens after the last block boundary
+  rc |= fused(1, 0, 90, 12, 1, 64, 64, 70);   // no full block
+  rc |= fused(1, 2, 64, 100, 1, 128, 64);     // suffixes in two parts
+  rc |= fused(1, 8, 64, 16, 2, 128, 128);     // backward in the kernel that carries dS once, suffixes as extra stops
+  rc |= plain(1, 530, 2, 128, 128, false);    // the same kernel without suffixes, ragged last chunk
+  rc |= checkpointed(1, 600, 2, 128);         // ... with the forward's checkpoints
   rc |= decode(2, 3, 64, 128);
   rc |= decode(1, 1, 256, 256);
   rc |= rotary(3, 11, 2, 64, true);           // last workgroup partly idle
