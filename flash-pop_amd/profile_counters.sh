@@ -24,4 +24,5 @@ CMD=$COPY run copy_write --pmc WRITE_SIZE
 # the model-level step of benchmark configuration 5 (12-layer harness around the ops): which kernels its time goes to
 MODEL="python3 $R/bench.py --steps 10 --warmup 2 --spin-up 0 --no-cpu --no-pop --no-long --no-layer"
 CMD=$MODEL run model_trace --kernel-trace --stats
+rm -f "$O/model_trace/r_kernel_trace.csv"   # tens of MB, one line per launch; the per-kernel statistics beside it are what is summarised
 echo "done: $O"
