@@ -158,7 +158,7 @@ def gpu_leg(args):
             "launch_ms": round(bwd_ms, 4),
             "algorithmic_bytes_per_launch": b_bwd,
             # the other launch of a step and the step as a whole, priced the same way
-            "forward_kernel": "retention_pass_ws_kernel<128, 0, 1>",
+            "forward_kernel": "retention_pass_ws_kernel<128, 1, 1> (the forward pass, leaving its state every 512 tokens for the backward)",
             "forward_launch_ms": round(fwd_ms, 4),
             "forward_algorithmic_bytes_per_launch": b_fwd,
             "forward_achieved": round(fwd_gbs, 1),
@@ -184,10 +184,10 @@ def gpu_leg(args):
             o_s, _ = fused_chunk_retention(*sleaves, starts, decays)
             return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
 
-        for _ in range(max(2, args.warmup // 4)):
+        for _ in range(max(5, args.warmup // 2)):
             pop_step()
         torch.cuda.synchronize()
-        n = max(3, args.steps // 4)
+        n = max(12, args.steps // 4)
         t0 = time.perf_counter()
         for _ in range(n):
             pop_step()
@@ -199,7 +199,7 @@ def gpu_leg(args):
             o, o_s, _ = flash_pop_retention_with_suffixes(*leaves, s, decays, block, *sleaves)
             return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
 
-        for _ in range(max(2, args.warmup // 4)):
+        for _ in range(max(5, args.warmup // 2)):
             fused_step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -236,10 +236,10 @@ def gpu_leg(args):
             o, S = fused_chunk_retention(*l3, dec3)
             return torch.autograd.grad([o, S], l3, [d_o3, d_s3])
 
-        for _ in range(max(2, args.warmup // 4)):
+        for _ in range(max(5, args.warmup // 2)):
             long_step()
         torch.cuda.synchronize()
-        n = max(3, args.steps // 4)
+        n = max(12, args.steps // 4)
         t0 = time.perf_counter()
         for _ in range(n):
             long_step()

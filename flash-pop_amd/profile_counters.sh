@@ -11,10 +11,12 @@ R=$(cd "$(dirname "$0")/.." && pwd)
 mkdir -p "$1"
 O=$(cd "$1" && pwd)
 cd /tmp && export TMPDIR=/tmp
+# the trace run keeps bench.py's spin-up so that its durations are those of settled clocks; the counter runs skip it
+TRACE="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu --no-long --no-model"
 BENCH="python3 $R/bench.py --steps 8 --warmup 4 --spin-up 0 --no-cpu --no-long --no-model"
 COPY="python3 $R/bench.py --copy-calibration"
 run() { name=$1; shift; timeout -s KILL 120 rocprofv3 "$@" --output-format csv -d "$O/$name" -o r -- $CMD > "$O/$name.log" 2>&1; }
-CMD=$BENCH run trace --kernel-trace --stats
+CMD=$TRACE run trace --kernel-trace --stats
 CMD=$BENCH run sq1 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_INSTS_LDS SQ_INSTS_SALU SQ_WAIT_INST_LDS
 CMD=$BENCH run sq2 --pmc SQ_ACTIVE_INST_VALU SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_WAIT_INST_ANY SQ_WAIT_ANY SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU_MFMA_MOPS_BF16
 CMD=$BENCH run fetch --pmc FETCH_SIZE
