@@ -34,16 +34,24 @@ FP_DEVICE void rotary_qk(const RotaryArgs& p) {
     const uint16_t* src = which ? p.k_in : p.q_in;
     uint16_t* dst = which ? p.k_out : p.q_out;
     if (!src) continue;
-    for (int h = 0; h < p.H; ++h) {
-      const size_t at = at0 + (size_t)h * p.d;
-      const u32x4 v = ld128(src + at);
-      u32x4 o;
+    // four heads at a time, their loads issued before the first is used
+    for (int h0 = 0; h0 < p.H; h0 += 4) {
+      u32x4 v[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float e = bf16_elem(v, 2 * j), d = bf16_elem(v, 2 * j + 1);
-        o[j] = fprt::pack_bf16x2(e * cs[j] - d * sn[j], d * cs[j] + e * sn[j]);
+      for (int u = 0; u < 4; ++u) {
+        if (h0 + u < p.H) v[u] = ld128(src + at0 + (size_t)(h0 + u) * p.d);
       }
-      st128(dst + at, o);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (h0 + u >= p.H) break;
+        u32x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float e = bf16_elem(v[u], 2 * j), d = bf16_elem(v[u], 2 * j + 1);
+          o[j] = fprt::pack_bf16x2(e * cs[j] - d * sn[j], d * cs[j] + e * sn[j]);
+        }
+        st128(dst + at0 + (size_t)(h0 + u) * p.d, o);
+      }
     }
   }
 }

@@ -261,5 +261,3 @@ def test_gated_group_norm(emu_lib, rows, H, dv):
     d_r_ref, d_g_ref = hp.oracle_gated_norm_grads(r, gate, d_out)
     hp.assert_close(d_r, d_r_ref, "d_r")
     hp.assert_close(d_g, d_g_ref, "d_g")
-
-

@@ -400,5 +400,3 @@ def test_non_finite_future_keys_do_not_reach_earlier_outputs():
     torch.cuda.synchronize()
     assert torch.isfinite(o_bad[:, :t0].float()).all()
     assert torch.equal(o_bad[:, :t0], o_clean)
-
-
