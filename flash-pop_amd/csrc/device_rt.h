@@ -37,7 +37,9 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 FP_DEVICE float exp2_approx(float x) { return __builtin_amdgcn_exp2f(x); }
 // full-precision elementary functions for the elementwise kernels
 FP_DEVICE void sincos_f32(float x, float& s, float& c) { sincosf(x, &s, &c); }
-FP_DEVICE float exp_f32(float x) { return expf(x); }
+// 1 / (1 + e^-x) from the hardware's 2^x and reciprocal (v_exp_f32, v_rcp_f32: ~1 ulp each; 0 and 1
+// at the far ends, where e^-x overflows or vanishes)
+FP_DEVICE float sigmoid_f32(float x) { return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504f * x)); }
 FP_DEVICE float rsqrt_f32(float x) { return 1.0f / sqrtf(x); }
 // value held by lane (this lane ^ mask) of the wave; every lane of the wave has to call it
 FP_DEVICE float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }

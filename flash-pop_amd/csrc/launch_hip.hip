@@ -284,7 +284,8 @@ int launched(const char** err) {
 
 }  // namespace
 
-int fpk_launch_rotary(const fpk::RotaryArgs& a, void* stream, const char** err) {
+int fpk_launch_rotary(const fpk::RotaryArgs& args, void* stream, const char** err) {
+  fpk::RotaryArgs a = args;
   long long blocks = 0;
   if (const char* why = fpk::plan_rotary(a, blocks)) {
     *err = why;

@@ -13,13 +13,18 @@
 namespace fpk {
 
 // ------------------------------------------------------------------------------------------
-// One thread: 8 adjacent features (4 rotation pairs) of one token, for every head of q and k.
+// One thread: 8 adjacent features (4 rotation pairs) of one token, for p.heads_per_thread heads of
+// q and k (all of them when there are plenty of tokens: the sines and cosines are then computed
+// once per token; a single decode token is spread over more threads instead of more loop trips).
 FP_DEVICE void rotary_qk(const RotaryArgs& p) {
-  const int opr = p.d / 8;                                   // threads per token
+  const int opr = p.d / 8;                                   // threads per token and head group
+  const int hgroups = (p.H + p.heads_per_thread - 1) / p.heads_per_thread;
   const long long unit = (long long)fprt::block_index() * LAYER_THREADS + fprt::thread_index();
-  const long long row = unit / opr;
+  const long long row = unit / (opr * hgroups);
   if (row >= (long long)p.B * p.T) return;
   const int oc = (int)(unit % opr);
+  const int h_first = (int)((unit / opr) % hgroups) * p.heads_per_thread;
+  const int h_end = h_first + p.heads_per_thread < p.H ? h_first + p.heads_per_thread : p.H;
   const int b = (int)(row / p.T), t = (int)(row % p.T);
   const float pos = (float)((p.start ? p.start[b] : p.start0) + t);
   float sn[4], cs[4];
@@ -35,15 +40,15 @@ FP_DEVICE void rotary_qk(const RotaryArgs& p) {
     uint16_t* dst = which ? p.k_out : p.q_out;
     if (!src) continue;
     // four heads at a time, their loads issued before the first is used
-    for (int h0 = 0; h0 < p.H; h0 += 4) {
+    for (int h0 = h_first; h0 < h_end; h0 += 4) {
       u32x4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        if (h0 + u < p.H) v[u] = ld128(src + at0 + (size_t)(h0 + u) * p.d);
+        if (h0 + u < h_end) v[u] = ld128(src + at0 + (size_t)(h0 + u) * p.d);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        if (h0 + u >= p.H) break;
+        if (h0 + u >= h_end) break;
         u32x4 o;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -105,7 +110,7 @@ FP_DEVICE void gated_norm_fwd(const GatedNormArgs& p) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float g = bf16_elem(gv, e);
-    const float gate = round_bf16(g / (1.f + fprt::exp_f32(-g)));
+    const float gate = round_bf16(g * fprt::sigmoid_f32(g));
     y[e] = round_bf16(st.dev[e] * st.rstd) * gate;
   }
   u32x4 o;
@@ -132,7 +137,7 @@ FP_DEVICE void gated_norm_bwd(const GatedNormArgs& p) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float g = bf16_elem(gv, e), dy = bf16_elem(dv_, e);
-    const float sig = 1.f / (1.f + fprt::exp_f32(-g));
+    const float sig = fprt::sigmoid_f32(g);
     nh[e] = st.dev[e] * st.rstd;
     dn[e] = dy * round_bf16(g * sig);
     dg[e] = dy * round_bf16(nh[e]) * (sig * (1.f + g * (1.f - sig)));
@@ -157,11 +162,16 @@ FP_DEVICE void gated_norm_bwd(const GatedNormArgs& p) {
 // ------------------------------------------------------------------------------------------
 // Host side: argument checks and grid sizes, shared by the GPU launcher and the CPU test harness.
 // Return nullptr if the launch is valid (and the number of workgroups in `blocks`), else the reason.
-inline const char* plan_rotary(const RotaryArgs& a, long long& blocks) {
+// (chooses a.heads_per_thread)
+inline const char* plan_rotary(RotaryArgs& a, long long& blocks) {
   if (a.B < 1 || a.T < 1 || a.H < 1 || a.d < 8 || a.d % 8 != 0) return "rotary: B, T, H >= 1 and d a multiple of 8 expected";
   if (!a.q_in || !a.q_out || !a.theta || (a.k_in == nullptr) != (a.k_out == nullptr)) return "rotary: null pointer";
   if (a.sign != 1.f && a.sign != -1.f) return "rotary: sign must be +1 or -1";
-  const long long units = (long long)a.B * a.T * (a.d / 8);
+  // fewer than two waves per compute unit's worth of token threads: one head per thread, so that a
+  // decode step's few tokens do not walk all heads in a loop of dependent loads
+  const long long token_threads = (long long)a.B * a.T * (a.d / 8);
+  a.heads_per_thread = token_threads >= (1 << 15) ? a.H : 1;
+  const long long units = token_threads * ((a.H + a.heads_per_thread - 1) / a.heads_per_thread);
   blocks = (units + LAYER_THREADS - 1) / LAYER_THREADS;
   return blocks > 0x7fffffffLL ? "rotary: too many tokens for one launch" : nullptr;
 }

@@ -152,6 +152,7 @@ struct RotaryArgs {
   long long start0;
   int B, T, H, d;
   float sign;
+  int heads_per_thread;    // set by plan_rotary: all H, or fewer when there are too few tokens to fill the device
 };
 
 // Per-head normalisation of the retention output followed by the swish gate:

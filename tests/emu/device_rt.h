@@ -78,7 +78,7 @@ FP_DEVICE uint32_t pack_bf16x2(float lo, float hi) {
 
 FP_DEVICE float exp2_approx(float x) { return std::exp2(x); }
 FP_DEVICE void sincos_f32(float x, float& s, float& c) { s = std::sin(x); c = std::cos(x); }
-FP_DEVICE float exp_f32(float x) { return std::exp(x); }
+FP_DEVICE float sigmoid_f32(float x) { return 1.0f / (1.0f + std::exp(-x)); }
 FP_DEVICE float rsqrt_f32(float x) { return 1.0f / std::sqrt(x); }
 
 FP_DEVICE void sched_fence() {}

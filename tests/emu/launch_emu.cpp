@@ -145,7 +145,8 @@ int fpk_launch_decode(const fpk::DecodeArgs& a, void* /*stream*/, const char** e
   return run_grid(fpk::DECODE_THREADS, a.B * a.H, fpk::decode_lds_bytes(a.dv), [&](char* l) { fpk::decode_step(a, l); });
 }
 
-int fpk_launch_rotary(const fpk::RotaryArgs& a, void* /*stream*/, const char** err) {
+int fpk_launch_rotary(const fpk::RotaryArgs& args, void* /*stream*/, const char** err) {
+  fpk::RotaryArgs a = args;
   long long blocks = 0;
   if (const char* why = fpk::plan_rotary(a, blocks)) {
     *err = why;

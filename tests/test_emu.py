@@ -225,7 +225,8 @@ def test_gamma_one_and_tiny(emu_lib):
     hp.assert_close(S, S_ref, "S")
 
 
-@pytest.mark.parametrize("B,T,H,d,vec", [(2, 37, 3, 64, False), (3, 5, 2, 128, True), (1, 300, 1, 8, False)])
+@pytest.mark.parametrize("B,T,H,d,vec", [(2, 37, 3, 64, False), (3, 5, 2, 128, True), (1, 300, 1, 8, False),
+                                         (1, 4096, 5, 64, False)])   # enough tokens for one thread to take all heads
 def test_rotary(emu_lib, B, T, H, d, vec):
     """Rotation of q and k (also q alone, in place, and back) against the oracle."""
     g = torch.Generator().manual_seed(d + T)
@@ -234,11 +235,18 @@ def test_rotary(emu_lib, B, T, H, d, vec):
     start = torch.tensor([7, 4000, 123456][:B]) if vec else 1000
     pos = (start[:, None] if vec else start) + torch.arange(T)[None]
     rq, rk = hp.raw_rotary(emu_lib, q, k, theta, start)
-    assert torch.equal(rq, oracle.rotary(q, pos, theta)) and torch.equal(rk, oracle.rotary(k, pos, theta))
+
+    def same(got, ref):
+        """Equal, or (libm's and torch's sine may differ in the last place of an fp32 angle of a few
+        thousand radians) a handful of elements apart by one bf16 step."""
+        diff = (got.float() - ref.float()).abs()
+        return bool((diff > 0).float().mean() < 1e-4) and bool((diff <= ref.float().abs() * 2.0 ** -7 + 1e-5).all())
+
+    assert same(rq, oracle.rotary(q, pos, theta)) and same(rk, oracle.rotary(k, pos, theta))
     only_q, none = hp.raw_rotary(emu_lib, q, None, theta, start)
     assert none is None and torch.equal(only_q, rq)
     back_q, back_k = hp.raw_rotary(emu_lib, rq, rk, theta, start, inverse=True)
-    assert torch.equal(back_q, oracle.rotary(rq, pos, theta, inverse=True))
+    assert same(back_q, oracle.rotary(rq, pos, theta, inverse=True))
     hp.assert_close(back_k, k.float(), "round trip")
     q2, k2 = q.clone(), k.clone()
     hp.raw_rotary(emu_lib, q2, k2, theta, start, in_place=True)
