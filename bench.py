@@ -184,6 +184,9 @@ def gpu_leg(args):
             o_s, _ = fused_chunk_retention(*sleaves, starts, decays)
             return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
 
+        # (the inputs of this leg were made on the host: the device idled meanwhile and its clocks fell back)
+        if args.spin_up > 0:
+            spin_up(pop_step, args.spin_up)
         for _ in range(max(5, args.warmup // 2)):
             pop_step()
         torch.cuda.synchronize()
@@ -236,6 +239,8 @@ def gpu_leg(args):
             o, S = fused_chunk_retention(*l3, dec3)
             return torch.autograd.grad([o, S], l3, [d_o3, d_s3])
 
+        if args.spin_up > 0:
+            spin_up(long_step, args.spin_up)
         for _ in range(max(5, args.warmup // 2)):
             long_step()
         torch.cuda.synchronize()

@@ -293,8 +293,12 @@ int plan_segments(const Shape& s, int tiles) {
   }
   return best;
 }
-int plan_forward(const Shape& s) { return plan_segments(s, s.dv / fpk::BV); }
-int plan_backward(const Shape& s) { return plan_segments(s, (s.dk < s.dv ? s.dk : s.dv) / fpk::BV); }
+// Forward and backward cut a sequence the same way (the backward's narrowest pass has the fewest
+// column tiles and decides), so that the states the forward leaves at the start of every segment
+// are the ones the backward's dq pass needs.
+int plan_split(const Shape& s) { return plan_segments(s, (s.dk < s.dv ? s.dk : s.dv) / fpk::BV); }
+int plan_forward(const Shape& s) { return plan_split(s); }
+int plan_backward(const Shape& s) { return plan_split(s); }
 
 size_t workspace_bytes(const Shape& s, int segments) {
   return segments > 1 ? 2 * sizeof(uint16_t) * (size_t)s.B * segments * s.H * s.dk * s.dv : 0;
@@ -354,16 +358,18 @@ int forward_split(const Shape& s, int segments, const void* q, const void* k, co
 
 int backward_split(const Shape& s, int segments, const void* q, const void* k, const void* v, const void* s0,
                    const double* decays, const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_,
-                   void* d_s0, void* workspace, void* stream) {
+                   void* d_s0, void* workspace, bool states_kept, void* stream) {
   const Shape seg = segment_shape(s, segments);
   const Workspace w = carve(workspace, s, segments);
   const float sc = 1.0f / std::sqrt((float)s.dk);
   fpk::PassArgs a;
   int rc;
 
-  // S at the start of every segment, then dq
-  if ((rc = contributions(seg, decays, k, v, 0, w, stream)) != FP_OK) return rc;
-  if ((rc = scan(s, segments, decays, w, s0, nullptr, 0, stream)) != FP_OK) return rc;
+  // S at the start of every segment (unless the forward's are still there), then dq
+  if (!states_kept) {
+    if ((rc = contributions(seg, decays, k, v, 0, w, stream)) != FP_OK) return rc;
+    if ((rc = scan(s, segments, decays, w, s0, nullptr, 0, stream)) != FP_OK) return rc;
+  }
   fill_common(a, seg, decays);
   a.X = in(d_o); a.W = in(v); a.Z = in(k); a.Y = out(dq);
   a.R0 = w.start;
@@ -571,7 +577,8 @@ int fp_retention_fwd_split_static(const void* q, const void* k, const void* v, c
 
 int fp_retention_bwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
                            const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B,
-                           int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes_given, void* stream) {
+                           int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes_given,
+                           int forward_states_kept, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
   if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
@@ -579,7 +586,8 @@ int fp_retention_bwd_split(const void* q, const void* k, const void* v, const vo
   const int segments = plan_backward(s);
   if (int rc = check_workspace(s, segments, workspace, workspace_bytes_given)) return rc;
   if (segments <= 1) return backward(s, q, k, v, s0, head_decays, d_o, d_s_out, nullptr, 0, dq, dk_, dv_, d_s0, stream);
-  return backward_split(s, segments, q, k, v, s0, head_decays, d_o, d_s_out, dq, dk_, dv_, d_s0, workspace, stream);
+  return backward_split(s, segments, q, k, v, s0, head_decays, d_o, d_s_out, dq, dk_, dv_, d_s0, workspace,
+                        forward_states_kept != 0, stream);
 }
 
 int fp_pop_retention_fwd(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,

@@ -23,7 +23,7 @@ SIGNATURES = {
     "fp_retention_workspace_bytes": [_I, _I, _I, _I, _I],
     "fp_retention_fwd_split": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
     "fp_retention_fwd_split_static": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _P],
-    "fp_retention_bwd_split": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
+    "fp_retention_bwd_split": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _Z, _I, _P],
     "fp_pop_retention_fwd": [_P, _P, _P, _P, _D, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "fp_pop_retention_bwd": [_P, _P, _P, _P, _D, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "fp_pop_fused_fwd": [_P] * 7 + [_D] + [_P] * 3 + [_I] * 7 + [_P],

@@ -57,8 +57,10 @@ def _workspace(lib, shape, device):
 
 
 def retention_fwd(q, k, v, s, decays, shape, for_backward=False):
-    """-> (o, s_out, checkpoints or None, checkpoint interval).  With `for_backward` the forward
-    also leaves the states that make the backward cheaper, where the library says they pay."""
+    """-> (o, s_out, states or None, checkpoint interval).  With `for_backward` the forward also
+    leaves the states that make the backward cheaper, where the library says they pay: checkpoints
+    every `interval` tokens, or (interval 0) the workspace of a forward that cut its sequences into
+    segments, which holds the state at the start of every segment."""
     refuse_capture("retention_fwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
@@ -83,7 +85,7 @@ def retention_fwd(q, k, v, s, decays, shape, for_backward=False):
             rc = lib.fp_retention_fwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(o),
                                             _ptr(s_out), B, T, H, dk, dv, _ptr(ws), ws.numel(), _stream())
     _lib.check(lib, rc)
-    return o, s_out, ckpt, every
+    return o, s_out, ckpt if ckpt is not None else (ws if for_backward else None), every
 
 
 def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
@@ -101,7 +103,7 @@ def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
 
 def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0, ckpt=None, every=0):
     """Gradients for both ops; block_size is None for the plain op.  ckpt, every: what retention_fwd
-    left for this call."""
+    left for this call (every = 0 with a tensor: the forward's workspace)."""
     refuse_capture("retention_bwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
@@ -111,15 +113,16 @@ def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size,
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     d_s0 = torch.empty((B, H, dk, dv), dtype=q.dtype, device=q.device) if want_ds0 else None
     with torch.cuda.device(q.device):
-        ws = _workspace(lib, shape, q.device) if block_size is None else None
-        if ckpt is not None and block_size is None:
+        kept = ckpt is not None and every == 0      # the workspace of a forward that cut its sequences
+        ws = ckpt if kept else _workspace(lib, shape, q.device) if block_size is None else None
+        if ckpt is not None and not kept and block_size is None:
             rc = lib.fp_retention_bwd_ckpt(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                            _ptr(d_s_out), _ptr(ckpt), every, _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0),
                                            B, T, H, dk, dv, _stream())
         elif ws is not None:
             rc = lib.fp_retention_bwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                             _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
-                                            _ptr(ws), ws.numel(), _stream())
+                                            _ptr(ws), ws.numel(), int(kept), _stream())
         elif block_size is None:
             rc = lib.fp_retention_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                       _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,

@@ -83,16 +83,23 @@ int fp_retention_bwd_ckpt(const void* q, const void* k, const void* v, const voi
  * reference, whose kernels also walk a sequence serially (fused_chunk_fwd.py:95-187).
  *   fp_retention_workspace_bytes  scratch bytes the two calls need for this shape on the current
  *                                 device; 0 means they would not cut (and accept workspace = NULL)
- *   workspace                     device memory, 16-byte aligned, at least that many bytes; its
- *                                 contents are undefined afterwards, and two calls that share it
- *                                 must be ordered by their stream */
+ *   workspace                     device memory, 16-byte aligned, at least that many bytes; two calls
+ *                                 that share it must be ordered by their stream.  After
+ *                                 fp_retention_fwd_split it holds the state at the start of every
+ *                                 segment, which the backward needs too:
+ *   forward_states_kept           nonzero: `workspace` is the buffer fp_retention_fwd_split was given
+ *                                 for the same q, k, v, s0 and decays and nothing has written to it
+ *                                 since; the backward then skips recomputing those states (one pass
+ *                                 over k and v).  0: the workspace holds nothing of use.
+ *                                 Either way its contents are undefined after the backward. */
 size_t fp_retention_workspace_bytes(int B, int T, int H, int dk, int dv);
 int fp_retention_fwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
                            void* o, void* s_out, int B, int T, int H, int dk, int dv, void* workspace,
                            size_t workspace_bytes, void* stream);
 int fp_retention_bwd_split(const void* q, const void* k, const void* v, const void* s0, const double* head_decays,
                            const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, int B,
-                           int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes, void* stream);
+                           int T, int H, int dk, int dv, void* workspace, size_t workspace_bytes,
+                           int forward_states_kept, void* stream);
 
 /* fp_retention_fwd_split without a workspace argument and without any allocation.  It has no
  * counterpart in the reference; it is for callers that cannot allocate device memory at the call:

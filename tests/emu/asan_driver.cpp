@@ -41,7 +41,8 @@ int plain(int B, int T, int H, int dk, int dv, bool split) {
     const size_t wb = fp_retention_workspace_bytes(B, T, H, dk, dv);
     void* ws = wb ? aligned_alloc(16, wb) : nullptr;
     rc = fp_retention_fwd_split(q, k, v, s, dec.data(), o, so, B, T, H, dk, dv, ws, wb, nullptr);
-    if (!rc) rc = fp_retention_bwd_split(q, k, v, s, dec.data(), dO, dS, dq, dk_, dv_, ds0, B, T, H, dk, dv, ws, wb, nullptr);
+    if (!rc) rc = fp_retention_bwd_split(q, k, v, s, dec.data(), dO, dS, dq, dk_, dv_, ds0, B, T, H, dk, dv, ws, wb, 1, nullptr);
+    if (!rc) rc = fp_retention_bwd_split(q, k, v, s, dec.data(), dO, dS, dq, dk_, dv_, ds0, B, T, H, dk, dv, ws, wb, 0, nullptr);
     free(ws);
     return done(rc, "split", B, T, H, dk, dv, (int)wb);
   }

@@ -243,9 +243,9 @@ def raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot, stream=None, want_ds
     return outs + [ds0]
 
 
-def raw_split_fwd(lib, q, k, v, s, decays, stream=None):
+def raw_split_fwd(lib, q, k, v, s, decays, stream=None, keep_workspace=False):
     """fp_retention_fwd_split with a workspace of exactly the size the library asks for.
-    Returns (o, s_out, workspace bytes)."""
+    Returns (o, s_out, workspace bytes[, the workspace])."""
     B, T, H, dk = q.shape
     dv = v.shape[3]
     nbytes = lib.fp_retention_workspace_bytes(B, T, H, dk, dv)
@@ -254,19 +254,23 @@ def raw_split_fwd(lib, q, k, v, s, decays, stream=None):
     S = torch.full((B, H, dk, dv), float("nan"), dtype=BF16, device=q.device)
     _check(lib, lib.fp_retention_fwd_split(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(o), _p(S), B, T, H, dk, dv,
                                            _p(ws) if nbytes else None, nbytes, stream))
+    if keep_workspace:
+        return o, S, nbytes, ws
     return o, S, nbytes
 
 
-def raw_split_bwd(lib, q, k, v, s, decays, d_o, d_s, stream=None):
+def raw_split_bwd(lib, q, k, v, s, decays, d_o, d_s, stream=None, forward_workspace=None):
+    """forward_workspace: the buffer raw_split_fwd(keep_workspace=True) returned for the same inputs;
+    the backward then starts from the segment states the forward left in it."""
     B, T, H, dk = q.shape
     dv = v.shape[3]
     nbytes = lib.fp_retention_workspace_bytes(B, T, H, dk, dv)
-    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+    ws = forward_workspace if forward_workspace is not None else torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
     nan = lambda *shape: torch.full(shape, float("nan"), dtype=BF16, device=q.device)
     dq, dk_, dv_, ds0 = nan(*q.shape), nan(*k.shape), nan(*v.shape), nan(B, H, dk, dv)
     _check(lib, lib.fp_retention_bwd_split(_p(q), _p(k), _p(v), _p(s), _dec(decays), _p(d_o), _p(d_s), _p(dq), _p(dk_),
                                            _p(dv_), _p(ds0), B, T, H, dk, dv, _p(ws) if nbytes else None, nbytes,
-                                           stream))
+                                           int(forward_workspace is not None), stream))
     return dq, dk_, dv_, ds0
 
 

@@ -93,7 +93,7 @@ def test_new_entry_points_check_their_arguments(lib):
     assert lib.fp_retention_workspace_bytes(0, 64, 2, 64, 64) == 0
     assert lib.fp_retention_workspace_bytes(1, 64, 2, 96, 64) == 0
     assert lib.fp_retention_fwd_split(null, p, p, null, dec, p, null, 1, 8, 2, 64, 64, null, 0, None) == -1
-    assert lib.fp_retention_bwd_split(p, p, p, null, dec, null, null, p, p, p, null, 1, 8, 2, 64, 64, null, 0, None) == -1
+    assert lib.fp_retention_bwd_split(p, p, p, null, dec, null, null, p, p, p, null, 1, 8, 2, 64, 64, null, 0, 0, None) == -1
 
 
 def test_new_python_wrappers_refuse_cpu_tensors():

@@ -112,6 +112,10 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     dq, dk_, dv_, ds0 = hp.raw_split_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
     o_ref, S_ref, (gq, gk, gv, gs) = hp.oracle_plain(q, k, v, s, decays, d_o, d_s)
     _check_all([("o", o, o_ref), ("S", S, S_ref), ("dq", dq, gq), ("dk", dk_, gk), ("dv", dv_, gv), ("ds0", ds0, gs)])
+    # the backward that starts from the segment states the forward left in its workspace: same bits
+    o2, S2, _, ws = hp.raw_split_fwd(emu_lib, q, k, v, s, decays, keep_workspace=True)
+    again = hp.raw_split_bwd(emu_lib, q, k, v, s, decays, d_o, d_s, forward_workspace=ws)
+    assert torch.equal(o2, o) and all(torch.equal(a, b) for a, b in zip(again, (dq, dk_, dv_, ds0)))
 
 
 @pytest.mark.parametrize("B,nblk,block,Ls,H,state_std", [

@@ -297,6 +297,11 @@ def test_split_entry_points_long_sequence_few_streams(B, T, H, dk, dv):
     hp.assert_close(o, o1.float(), "o vs unsplit", head_dim=2)
     for n, g, g1 in zip(names, grads, grads1):
         hp.assert_close(g, g1.float(), f"{n} vs unsplit", head_dim=1 if n == "ds0" else 2)
+    # the backward that starts from the segment states the forward left in its workspace: same bits
+    o2, S2, _, ws = hp.raw_split_fwd(lib, q, k, v, s, decays, keep_workspace=True)
+    again = hp.raw_split_bwd(lib, q, k, v, s, decays, d_o, d_s, forward_workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o) and all(torch.equal(x, y) for x, y in zip(again, grads))
     # workspace checks happen before any launch
     p, dec = hp._p, hp._dec(decays)
     small = torch.empty(nbytes - 16, dtype=torch.uint8, device=DEV)
