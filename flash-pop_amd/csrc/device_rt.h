@@ -74,6 +74,9 @@ FP_DEVICE BufView make_buf(const void* base, uint32_t nbytes) {
 FP_DEVICE u32x4 buf_load128(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, off, 0, 0); }
 FP_DEVICE u32x2 buf_load64(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b64(b.rsrc, off, 0, 0); }
 FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, b.rsrc, off, 0, 0); }
+// the same with the non-temporal hint: data that nobody reads again soon need not stay in the caches
+FP_DEVICE u32x4 buf_load128_nt(BufView b, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, off, 0, 2); }
+FP_DEVICE void buf_store128_nt(BufView b, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, b.rsrc, off, 0, 2); }
 FP_DEVICE void buf_store64(BufView b, uint32_t off, u32x2 v) { __builtin_amdgcn_raw_buffer_store_b64(v, b.rsrc, off, 0, 0); }
 
 }  // namespace fprt

@@ -179,14 +179,17 @@ struct Sources {
   const void* ctx[N];
   const void* sfx[N];
 };
-template <int N>
+// ONCE: bit x set = tensor x is read by nobody else (non-temporal load)
+template <int N, int ONCE = 0>
 FP_DEVICE void load_tiles(const Common& k, const Sources<N>& src, const Item& it, u32x4 (&pf)[2 * N]) {
 #pragma unroll
   for (int x = 0; x < N; ++x) {
     const fprt::BufView v = item_view(k, src.ctx[x], src.sfx[x], it);
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-      pf[2 * x + u] = fprt::buf_load128(v, (uint32_t)(k.ld_row + 32 * u) * k.rowp + k.ld_piece * 16);
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t off = (uint32_t)(k.ld_row + 32 * u) * k.rowp + k.ld_piece * 16;
+      pf[2 * x + u] = ((ONCE >> x) & 1) ? fprt::buf_load128_nt(v, off) : fprt::buf_load128(v, off);
+    }
   }
 }
 template <int N>
@@ -206,7 +209,9 @@ FP_DEVICE void drain_tile(const Common& k, const uint16_t* tile, void* dst, void
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int row = k.ld_row + 32 * u;
-    fprt::buf_store128(v, (uint32_t)row * k.rowp + k.ld_piece * 16, ld128(tile + at(row, 8 * k.ld_piece)));
+    // non-temporal: the gradients are not read back here, and kept out of the caches they leave
+    // room for the rows that the other workgroup of the stream is about to read a second time
+    fprt::buf_store128_nt(v, (uint32_t)row * k.rowp + k.ld_piece * 16, ld128(tile + at(row, 8 * k.ld_piece)));
   }
 }
 
@@ -382,17 +387,17 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   const float wread_full1 = p.scale * fprt::exp2_approx((float)(CH - 1 - 32 - c) * lg);
   const float gL_full = fprt::exp2_approx((float)CH * lg);
 
-  const Sources<2> src_qg = {{p.q, p.dO}, {p.q_sfx, p.dO_sfx}};
+  const Sources<2> src_qg = {{p.q, p.dO}, {p.q_sfx, p.dO_sfx}};   // q: read by this workgroup only
   const Sources<2> src_kv = {{p.k, p.v}, {p.k_sfx, p.v_sfx}};
   const int nitems = item_count(k);
   Item cur = item_backward(k, 0), nxt = item_backward(k, 1), prev = cur;
   u32x4 pf_qg[4], pf_kv[4];
-  load_tiles<2>(k, src_qg, cur, pf_qg);
+  load_tiles<2, 1>(k, src_qg, cur, pf_qg);
   load_tiles<2>(k, src_kv, cur, pf_kv);
   load_state(k, Rt, p.ds_out ? p.ds_out + (size_t)stream * FB_D * FB_D : nullptr, false);
   stage_tiles<2>(k, TL, pf_qg);
   stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
-  load_tiles<2>(k, src_qg, nxt, pf_qg);
+  load_tiles<2, 1>(k, src_qg, nxt, pf_qg);
   load_tiles<2>(k, src_kv, nxt, pf_kv);
   fprt::block_sync();
   f32x16 racc[2];
@@ -406,6 +411,9 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   for (int it = 0; it < nitems; ++it) {
     const int L = cur.L;
     const bool sfx = SFX && cur.sfx;
+    // a suffix of at most 16 tokens lives in the first k-step of tokens and the first 32-token half:
+    // one score tile, one product each for the outputs and the state
+    const bool brief = sfx && L <= 16;
     const Item after = item_backward(k, it + 2);
     // ---- the previous item's outputs leave (nothing writes the staging tiles before the next barrier)
     if (it > 0) {
@@ -428,7 +436,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       };
       constexpr int AHEAD = 3;   // k-steps of operands in flight
       if (sfx) {   // no read-out: only the score tile
-        if (scores) {
+        if (scores && !(brief && rt != 0)) {
 #pragma unroll
           for (int t = 0; t < 8; ++t) {
             wf[t] = frag_cols(s_wrow, t);
@@ -479,6 +487,17 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     fprt::block_sync();
 
     // ---- stretch 2: Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]
+    if (brief) {
+      const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * rt), pq = ld128(xp_pass + lane * 8);
+      const u32x4 ua = frag_rows(Qs, tr_nat, 0, 32 * at_);
+      const u32x4 ub0 = frag_rows(Gs, tr_nat, 0, 32 * nt0), ub1 = frag_rows(Gs, tr_nat, 0, 32 * (nt0 + 1));
+      fprt::sched_fence();
+      acc[0] = fprt::mfma_32x32x16_bf16(za, pq, acc[0]);
+      const u32x4 wa = weigh(ua, wk0);
+      racc[0] = fprt::mfma_32x32x16_bf16(wa, ub0, racc[0]);
+      racc[1] = fprt::mfma_32x32x16_bf16(wa, ub1, racc[1]);
+      put_output(out, c, 32 * rt, g, acc[0]);
+    } else {
     {
       u32x4 za[4], pq0[4], pq1[2];
 #pragma unroll
@@ -530,6 +549,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
         fprt::sched_fence();
       }
     }
+    }
     // nobody reads this chunk's k and v tiles or the old copy of dS any more
     stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
     load_tiles<2>(k, src_kv, after, pf_kv);
@@ -539,7 +559,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
 
     // ---- stretch 3: every read of this chunk's q and dO tiles is done
     stage_tiles<2>(k, TL, pf_qg);
-    load_tiles<2>(k, src_qg, after, pf_qg);
+    load_tiles<2, 1>(k, src_qg, after, pf_qg);
     fprt::block_sync();
     prev = cur;
     cur = nxt;
@@ -639,11 +659,12 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     const bool fresh = !SFX && next >= 0 && next != chunk_of(it) + 1;   // the next chunk starts another segment
     const bool sfx = SFX && cur.sfx;
     const int L = cur.L;
+    const bool brief = sfx && L <= 16;   // as in the reverse workgroup: first k-step of tokens, first half only
     const Item after = item_of(it + 2);
     if (it > 0) drain_tile(k, OUT, p.dq, p.dq_sfx, prev);   // nothing writes the staging tile before the next barrier
     f32x16 acc[2];
     if constexpr (state_role) {
-      if (rt < 3) {
+      if (rt < 3 && !(brief && rt != 0)) {
         ScoreFrags sf;
         f32x16 sc = {0};
 #pragma unroll
@@ -661,6 +682,19 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
       // Y^T[n][i] = gamma^(i+1) sum_a R^T[n][a] X[i][a]
       acc[0] = f32x16{0};
       acc[1] = f32x16{0};
+      if (brief) {
+        u32x4 ra[8], x0[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          ra[t] = frag_cols(rrow, t);
+          x0[t] = frag_cols(xrow0, t);
+        }
+        fprt::sched_fence();
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][r] *= wread0;
+      } else {
       u32x4 ra[8], x0[8], x1[8];
       auto request = [&](int t) {
         ra[t] = frag_cols(rrow, t);
@@ -682,12 +716,18 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
         acc[0][r] *= wread0;
         acc[1][r] *= wread1;
       }
+      }
     }
     fprt::block_sync();
 
     if constexpr (!state_role) {
       // Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]; tokens j < 32 reach both halves (tiles (0,0), (0,1)),
       // the others only the second
+      if (brief) {
+        const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * rt), pq = ld128(XP + lane * 8);
+        acc[0] = fprt::mfma_32x32x16_bf16(za, pq, acc[0]);
+        put_output(OUT, c, 32 * rt, g, acc[0]);
+      } else {
       u32x4 za[4], pq1[4], pq0[2];
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) {
@@ -703,6 +743,7 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
       }
       put_output(OUT, c, 32 * rt, g, acc[0]);
       put_output(OUT, 32 + c, 32 * rt, g, acc[1]);
+      }
     } else if (!sfx) {
       // R[a][n] = gamma^L R + sum_j s gamma^(L-1-j) W[j][a] Z[j][n]
       const float gL = L == CH ? gL_full : fprt::exp2_approx((float)L * lg);

@@ -364,8 +364,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
       const bool live = c2.ok && !STATE;
       const fprt::BufView yv = fprt::make_buf(((SFX && c2.sfx) ? Ysg : Yg) + (live ? rowsB(c2) : 0),
                                               live ? (uint32_t)(c2.L - 1) * rowB + BV * 2 : 0u);
-      fprt::buf_store128(yv, yg_off, v0);
-      fprt::buf_store128(yv, yg_off + 16, v1);
+      // non-temporal: outputs are not read back by this launch and need not displace its inputs in the caches
+      fprt::buf_store128_nt(yv, yg_off, v0);
+      fprt::buf_store128_nt(yv, yg_off + 16, v1);
     };
 
     Chunk ck = first_chunk(slot), ck1 = chunk_after(ck), ckp = no_chunk;

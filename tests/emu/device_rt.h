@@ -131,5 +131,8 @@ FP_DEVICE void buf_store128(BufView b, uint32_t off, u32x4 v) {
 FP_DEVICE void buf_store64(BufView b, uint32_t off, u32x2 v) {
   if ((uint64_t)off + 8 <= b.nbytes) std::memcpy(const_cast<char*>(b.base) + off, &v, 8);
 }
+// the non-temporal forms differ only in how the device's caches treat the data
+FP_DEVICE u32x4 buf_load128_nt(BufView b, uint32_t off) { return buf_load128(b, off); }
+FP_DEVICE void buf_store128_nt(BufView b, uint32_t off, u32x4 v) { buf_store128(b, off, v); }
 
 }  // namespace fprt
