@@ -58,6 +58,9 @@ def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, 
     (1, 130, 2, 256, 128, 0.1),      # dk = 256
     (2, 2048, 4, 64, 128, 0.0),      # reference grads test shape (tests/test_fused_retention.py:240-282)
     (1, 70, 128, 64, 64, 0.1),       # the largest supported head count (decays down to 1 - 2^-132, i.e. 1.0)
+    (4, 1000, 16, 128, 128, 0.1),    # the backward that carries dS once, one checkpoint and a ragged stretch after it
+    (2, 513, 32, 128, 128, None),    # ... a one-token last chunk behind the only checkpoint, no state argument
+    (1, 4100, 64, 128, 128, 0.05),   # ... eight checkpoints, 64 heads
 ])
 def test_parity_sweep(B, T, H, dk, dv, state_std):
     run_plain(B, T, H, dk, dv, state_std, seed=T + dk)
