@@ -101,9 +101,11 @@ def pop_retention_fwd(q, k, v, s, decays, block_size, shape):
     return o, states
 
 
-def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0, ckpt=None, every=0):
+def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size, want_ds0, ckpt=None, every=0,
+                  states_kept=True):
     """Gradients for both ops; block_size is None for the plain op.  ckpt, every: what retention_fwd
-    left for this call (every = 0 with a tensor: the forward's workspace)."""
+    left for this call (every = 0 with a tensor: the forward's workspace, which still holds the
+    forward's segment states if `states_kept`)."""
     refuse_capture("retention_bwd")
     lib = _lib.load()
     B, T, H, dk, dv = shape
@@ -122,7 +124,7 @@ def retention_bwd(q, k, v, s, decays, shape, d_o, d_s_out, d_blocks, block_size,
         elif ws is not None:
             rc = lib.fp_retention_bwd_split(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                             _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,
-                                            _ptr(ws), ws.numel(), int(kept), _stream())
+                                            _ptr(ws), ws.numel(), int(kept and states_kept), _stream())
         elif block_size is None:
             rc = lib.fp_retention_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(s), _lib.decays_array(decays), _ptr(d_o),
                                       _ptr(d_s_out), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(d_s0), B, T, H, dk, dv,

@@ -22,6 +22,7 @@ class FusedChunkRetention(torch.autograd.Function):
         ctx.save_for_backward(q, k, v, s, ckpt)
         ctx.set_materialize_grads(False)   # an output nobody differentiates arrives as None, not as a tensor of zeros
         ctx.every = every
+        ctx.workspace_spent = False
         ctx.head_decays = tuple(head_decays)
         ctx.shape = shape
         return o, s_out
@@ -32,8 +33,12 @@ class FusedChunkRetention(torch.autograd.Function):
         if d_o is None:
             d_o = torch.zeros((*q.shape[:3], v.shape[3]), dtype=q.dtype, device=q.device)
         want_ds0 = s is not None and ctx.needs_input_grad[3]
+        # a forward that cut its sequences leaves its workspace (ctx.every == 0): the first backward
+        # starts from the states in it and overwrites them, a second one (retain_graph) recomputes them
+        kept = ckpt is not None and ctx.every == 0
         dq, dk, dv, d_s0 = _ops.retention_bwd(q, k, v, s, ctx.head_decays, ctx.shape, d_o, d_s_out, None, None, want_ds0,
-                                              ckpt, ctx.every)
+                                              ckpt, ctx.every, states_kept=kept and not ctx.workspace_spent)
+        ctx.workspace_spent = ctx.workspace_spent or kept
         return dq, dk, dv, d_s0, None
 
 

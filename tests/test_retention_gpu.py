@@ -196,6 +196,24 @@ def test_state_none_equals_zero_state_and_grad_flags():
     assert ql.grad is not None and ql.grad.shape == q.shape
 
 
+def test_backward_twice_through_a_cut_sequence():
+    """retain_graph on a shape that the op cuts into segments: the first backward consumes the segment
+    states the forward left in its workspace, the second has to recompute them.  Same gradients."""
+    from flash_pop_amd import fused_chunk_retention, _lib
+    B, T, H, dk, dv = 1, 4096, 2, 128, 128
+    assert _lib.load().fp_retention_workspace_bytes(B, T, H, dk, dv) > 0
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=31, state_std=0.1, device=DEV)
+    d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=32, device=DEV)
+    leaves = [t.requires_grad_() for t in (q, k, v, s)]
+    o, S = fused_chunk_retention(*leaves, decays)
+    first = torch.autograd.grad([o, S], leaves, [d_o, d_s], retain_graph=True)
+    second = torch.autograd.grad([o, S], leaves, [d_o, d_s])
+    torch.cuda.synchronize()
+    for name, a, b in zip(("dq", "dk", "dv", "ds0"), first, second):
+        assert torch.equal(a, b), name
+
+
 def test_gradient_through_the_final_state_only():
     """Only S is differentiated: the op receives no d_o (it is not materialised as zeros by autograd)
     and must behave as if it were zero; likewise for the POP op's block states."""
