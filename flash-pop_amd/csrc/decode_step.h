@@ -28,7 +28,8 @@ FP_DEVICE void decode_step(const DecodeArgs& p, char* lds) {
     v[e] = bf16_elem(vv, e);
     acc[e] = 0.f;
   }
-  for (int row = rg; row < p.dk; row += ngroups) {
+  // (dv = 192: 24 threads per row, 10 rows in flight, the last 16 threads idle)
+  for (int row = rg < ngroups ? rg : p.dk; row < p.dk; row += ngroups) {
     const float kr = p.scale * bf16_bits_to_float(reinterpret_cast<const u16_m*>(k)[row]);
     const float qr = bf16_bits_to_float(reinterpret_cast<const u16_m*>(q)[row]);
     const size_t at = mat + (size_t)row * p.dv + 8 * cg;
@@ -48,8 +49,10 @@ FP_DEVICE void decode_step(const DecodeArgs& p, char* lds) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += qr * s[e];
   }
+  if (rg < ngroups) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) part[rg * p.dv + 8 * cg + e] = acc[e];
+    for (int e = 0; e < 8; ++e) part[rg * p.dv + 8 * cg + e] = acc[e];
+  }
   fprt::block_sync();
   if (tid < p.dv) {
     float sum = 0.f;

@@ -43,7 +43,7 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-bool dim_ok(int d) { return d == 64 || d == 128 || d == 256; }
+bool dim_ok(int d) { return d == 64 || d == 128 || d == 192 || d == 256; }
 
 struct Shape {
   int B, T, H, dk, dv;
@@ -54,7 +54,7 @@ int check_shape(const Shape& s, const double* decays) {
   if (s.B < 1 || s.T < 1 || s.H < 1) return fail(FP_ERR_BAD_SHAPE, "B, T, H must be >= 1 (got %d, %d, %d)", s.B, s.T, s.H);
   if (s.H > fpk::MAX_HEADS) return fail(FP_ERR_BAD_SHAPE, "H = %d exceeds the supported maximum %d", s.H, fpk::MAX_HEADS);
   if (!dim_ok(s.dk) || !dim_ok(s.dv))
-    return fail(FP_ERR_UNSUPPORTED_DIM, "dk and dv must be 64, 128 or 256 (got dk=%d, dv=%d)", s.dk, s.dv);
+    return fail(FP_ERR_UNSUPPORTED_DIM, "dk and dv must be 64, 128, 192 or 256 (got dk=%d, dv=%d)", s.dk, s.dv);
   // per-tensor element counts are indexed with size_t in the kernel; the grid is an int
   // the kernels address one (batch, head) stream with 32-bit byte offsets
   const long long span = 2LL * s.T * s.H * (s.dk > s.dv ? s.dk : s.dv);

@@ -22,7 +22,7 @@ namespace fpk {
 
 constexpr int CH = 64;          // tokens per chunk
 constexpr int BV = 64;          // columns of Z / Y / R owned by one workgroup
-constexpr int MAX_HEADS = 128;
+constexpr int MAX_HEADS = 512;   // per-head decays travel in the kernel arguments (2 KB of the 4 KB a launch may carry)
 
 struct PassArgs {
   const uint16_t* X;

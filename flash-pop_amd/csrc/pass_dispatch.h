@@ -9,7 +9,7 @@
 namespace fpk {
 
 // Number of kernel instantiations `dispatch_pass` can pick from (its `slot` argument is below this).
-constexpr int PASS_KERNELS = 17;
+constexpr int PASS_KERNELS = 22;
 
 // Checks what the walks assume about `a` and chooses a.slots (workgroups per (head, column tile))
 // for a device with `compute_units` units.  Returns nullptr, or a message for the caller.
@@ -17,7 +17,7 @@ inline const char* plan_pass(PassArgs& a, int compute_units) {
   const bool blocks = a.block > 0 && (a.Bout || a.Bin);
   const bool narrow = a.dA == 64 || a.dA == 128;   // one visit per chunk
   const bool suffix = a.Ls > 0;
-  if (a.dA != 64 && a.dA != 128 && a.dA != 256) return "unsupported contraction width (dA must be 64, 128 or 256)";
+  if (a.dA != 64 && a.dA != 128 && a.dA != 192 && a.dA != 256) return "unsupported contraction width (dA must be 64, 128, 192 or 256)";
   if (a.dB < BV || a.dB % BV != 0) return "dB must be a multiple of 64";
   if (suffix) {
     // the C-ABI layer reports these to the caller in its own words
@@ -106,6 +106,13 @@ int dispatch_pass(const PassArgs& a, Run&& run) {
     if (a.state_only) return run.template go<128, WALK_STATE, 1>(7);
     if (multi) return run.template go<128, WALK_MULTI, 1>(8);
     return run.template go<128, WALK_PLAIN, 1>(9);
+  }
+  if (a.dA == 192) {   // three visits per chunk, 64 of the 192 contraction columns each
+    if (suffix_any) return run.template go<64, WALK_SUFFIX_ANY, 3>(17);
+    if (suffix) return run.template go<64, WALK_SUFFIX, 3>(18);
+    if (a.state_only) return run.template go<64, WALK_STATE, 3>(19);
+    if (blocks) return run.template go<64, WALK_BLOCKS, 3>(20);
+    return run.template go<64, WALK_PLAIN, 3>(21);
   }
   // dA = 256: two visits per chunk, 128 of the 256 contraction columns each
   if (suffix_any) return run.template go<128, WALK_SUFFIX_ANY, 2>(16);

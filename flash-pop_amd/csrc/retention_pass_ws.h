@@ -1,5 +1,5 @@
 // Wave-specialised retention pass (see pass_args.h for the recurrence): dA = 64 or 128 per visit,
-// dA = 256 in two visits per chunk (NH = 2 below).
+// dA = 256 in two visits per chunk, dA = 192 in three (NH below).
 //
 // One workgroup of 8 wave64 owns one (batch, head) stream and one 64-column slice of
 // Z / Y / R.  Hardware places waves w and w + 4 on the same SIMD, so every SIMD runs one
@@ -57,6 +57,30 @@ struct Half {
   static constexpr int value = H;
 };
 
+// Calls visit(part, it) for it = 0, 1, ... until it returns false, `part` being the visit's place in
+// the cycle of NH visits per chunk as a type (Half<it % NH>; with one visit per chunk the two
+// copies are the same code).  The LDS stage of a visit is it & 1, so a cycle of three is written
+// out over six visits.
+template <int NH, typename Visit>
+FP_DEVICE void walk_visits(Visit&& visit) {
+  if constexpr (NH == 3) {
+    for (int it = 0;; it += 6) {
+      if (!visit(Half<0>{}, it)) break;
+      if (!visit(Half<1>{}, it + 1)) break;
+      if (!visit(Half<2>{}, it + 2)) break;
+      if (!visit(Half<0>{}, it + 3)) break;
+      if (!visit(Half<1>{}, it + 4)) break;
+      if (!visit(Half<2>{}, it + 5)) break;
+    }
+  } else {
+    static_assert(NH == 1 || NH == 2, "one, two or three visits per chunk");
+    for (int it = 0;; it += 2) {
+      if (!visit(Half<0>{}, it)) break;
+      if (!visit(Half<1>{}, it + 1)) break;
+    }
+  }
+}
+
 // two 8-byte LDS reads that form one MFMA operand: tokens 16 kt + 4 g + {0..3} and + 8
 FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
   const u32x2 lo = ld64(p), hi = ld64(p + 8);
@@ -81,8 +105,8 @@ FP_DEVICE u32x4 ld_token_frag(const uint16_t* p) {
 //              the readout waves feed Z and do nothing else, X is not read and Y not written.
 enum Walk { WALK_PLAIN = 0, WALK_BLOCKS = 1, WALK_MULTI = 2, WALK_SUFFIX = 3, WALK_STATE = 4, WALK_SUFFIX_ANY = 5 };
 
-// NH = 2 handles a contraction width of 2 DA (p.dA = 256 with DA = 128) with the LDS footprint of
-// DA: every chunk is visited twice, once per half of the columns of X and W (of the rows of R).
+// NH > 1 handles a contraction width of NH * DA (p.dA = 256 as 2 x 128, p.dA = 192 as 3 x 64) with the
+// LDS footprint of DA: every chunk is visited NH times, once per part of the columns of X and W (of the rows of R).
 // Scores and read-out are sums over the contraction index, so the readout waves simply keep
 // accumulating across the two visits and convert, multiply by Z and store only after the second;
 // the state waves carry one set of accumulators per half and update the half being visited.
@@ -200,9 +224,9 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   };
   auto chunk_after = [&](const Chunk& ck) {
     if (!ck.ok) return ck;
-    if (NH == 2 && ck.h == 0) {   // the same chunk again, other half
+    if (NH > 1 && ck.h < NH - 1) {   // the same chunk again, next part of the contraction
       Chunk again = ck;
-      again.h = 1;
+      again.h = ck.h + 1;
       again.first = false;
       return again;
     }
@@ -251,7 +275,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   // [B, nblk + 1, Ls, H, dA]), resp. of this tile's columns in the dB-wide tensors: one 32 x 32 -> 64
   // bit multiply each (a tensor has fewer than 2^32 rows)
   const uint32_t headA = (uint32_t)h * p.dA * 2, headB = ((uint32_t)h * p.dB + (uint32_t)tile * BV) * 2;
-  auto rowsA = [&](const Chunk& ck) { return (size_t)ck.row * rowA + headA + (NH == 2 ? ck.h * DA * 2 : 0); };
+  auto rowsA = [&](const Chunk& ck) { return (size_t)ck.row * rowA + headA + (NH > 1 ? ck.h * DA * 2 : 0); };
   auto rowsB = [&](const Chunk& ck) { return (size_t)ck.row * rowB + headB; };
 
   if (!state_role) {
@@ -388,7 +412,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     auto iteration = [&](auto half, auto makes_c, auto both_c, int it) -> bool {
       constexpr int HF = decltype(half)::value;
       constexpr bool MAKES = decltype(makes_c)::value, BOTH = decltype(both_c)::value;
-      constexpr bool opens = NH == 1 || HF == 0, closes = NH == 1 || HF == 1;
+      constexpr bool opens = NH == 1 || HF == 0, closes = NH == 1 || HF == NH - 1;
       const int s = it & 1;
       const int L = ck.L;
       const Chunk ck2 = chunk_after(ck1);
@@ -522,20 +546,11 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     // Three copies of the loop, chosen once per wave: two live tiles and this wave makes one of
     // them; one live tile made by this wave; one live tile made by the partner.
     if (other_live) {
-      for (int it = 0;; it += 2) {
-        if (!iteration(Half<0>{}, Half<1>{}, Half<1>{}, it)) break;
-        if (!iteration(Half<1>{}, Half<1>{}, Half<1>{}, it + 1)) break;
-      }
+      walk_visits<NH>([&](auto part, int it) { return iteration(part, Half<1>{}, Half<1>{}, it); });
     } else if (makes_diag) {
-      for (int it = 0;; it += 2) {
-        if (!iteration(Half<0>{}, Half<1>{}, Half<0>{}, it)) break;
-        if (!iteration(Half<1>{}, Half<1>{}, Half<0>{}, it + 1)) break;
-      }
+      walk_visits<NH>([&](auto part, int it) { return iteration(part, Half<1>{}, Half<0>{}, it); });
     } else {
-      for (int it = 0;; it += 2) {
-        if (!iteration(Half<0>{}, Half<0>{}, Half<0>{}, it)) break;
-        if (!iteration(Half<1>{}, Half<0>{}, Half<0>{}, it + 1)) break;
-      }
+      walk_visits<NH>([&](auto part, int it) { return iteration(part, Half<0>{}, Half<0>{}, it); });
     }
     return;
   }
@@ -768,7 +783,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
   // it + 2 once they have gone into LDS.  Returns false after the last item.  `half` is the parity
   // of `it` as a type; with NH = 2 it is the half of R this visit updates.
   auto iteration = [&](auto half, int it) -> bool {
-    constexpr int HF = NH == 2 ? decltype(half)::value : 0;
+    constexpr int HF = NH > 1 ? decltype(half)::value : 0;
     constexpr bool closes = HF == NH - 1;   // the chunk is complete after this visit
     f32x16 (&racc_h)[NNW] = racc[HF];
     const int s = it & 1;
@@ -915,10 +930,7 @@ FP_DEVICE void retention_pass_ws(const PassArgs& p, const PassTensors& io, char*
     nxt = nn;
     return true;
   };
-  for (int it = 0;; it += 2) {
-    if (!iteration(Half<0>{}, it)) break;
-    if (!iteration(Half<1>{}, it + 1)) break;
-  }
+  walk_visits<NH>([&](auto part, int it) { return iteration(part, it); });
 }
 
 }  // namespace fpk

@@ -11,7 +11,7 @@
  *     [B,H,dk,dv]; block states [B, T/block_size, H, dk, dv]
  *   - head_decays is HOST memory: H doubles, gamma_h in (0, 1]
  *   - K is divided by sqrt(dk) inside (flash_pop/fused_retention/reference.py:57); Q is not scaled
- *   - dk, dv in {64, 128, 256}; 1 <= H <= 128; T >= 1; B >= 1
+ *   - dk, dv in {64, 128, 192, 256}; 1 <= H <= 512; T >= 1; B >= 1
  *   - the caller owns every buffer; the library allocates nothing and keeps no pointer
  *   - launches are asynchronous on `stream` (a hipStream_t, NULL = default stream)
  *   - returns 0 on success, a negative FP_ERR_* code otherwise; fp_last_error() then gives a

@@ -130,6 +130,7 @@ int main() {
   rc |= plain(2, 1, 1, 64, 64, false);        // single token
   rc |= plain(1, 65, 1, 64, 256, false);      // two visits per chunk, state read transposed
   rc |= plain(1, 130, 1, 256, 64, false);     // two visits per chunk, state as stored
+  rc |= plain(1, 100, 1, 192, 192, false);    // three visits per chunk
   rc |= plain(1, 512, 1, 64, 128, true);      // cut into segments (state-only walk, scan)
   rc |= pop(1, 287, 1, 64, 128, 144);
   rc |= pop(2, 28, 1, 64, 64, 15);

@@ -138,7 +138,7 @@ int fpk_launch_scan(const fpk::ScanArgs& a, void* /*stream*/, const char** err) 
 
 int fpk_launch_decode(const fpk::DecodeArgs& a, void* /*stream*/, const char** err) {
   if (a.B < 1 || a.H < 1 || a.H > fpk::MAX_HEADS || a.dk < 1 || a.dv < 8 || a.dv % 8 != 0 ||
-      fpk::DECODE_THREADS % (a.dv / 8) != 0 || a.dv > fpk::DECODE_THREADS || !a.q || !a.k || !a.v || !a.s_out || !a.o) {
+      a.dv > fpk::DECODE_THREADS || !a.q || !a.k || !a.v || !a.s_out || !a.o) {
     *err = "decode step: bad arguments";
     return 1;
   }

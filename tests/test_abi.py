@@ -64,8 +64,8 @@ def test_argument_checks_return_codes(lib):
     assert lib.fp_pop_retention_fwd(p, p, p, null, dec, p, p, *ok_dims, 0, None) == -2
     assert lib.fp_pop_retention_fwd(p, p, p, null, dec, p, null, *ok_dims, 4, None) == -1
     assert lib.fp_pop_retention_bwd(p, p, p, null, dec, p, p, p, p, null, null, *ok_dims, 4, None) == -1
-    big = (ctypes.c_double * 200)(*([0.9] * 200))
-    assert lib.fp_retention_fwd(p, p, p, null, big, p, null, 1, 8, 200, 64, 64, None) == -2
+    big = (ctypes.c_double * 513)(*([0.9] * 513))
+    assert lib.fp_retention_fwd(p, p, p, null, big, p, null, 1, 8, 513, 64, 64, None) == -2   # more than 512 heads
 
 
 def test_python_wrappers_refuse_cpu_tensors():

@@ -36,6 +36,10 @@ def _check_all(pairs):
     (1, 5, 3, 64, 64, 0.5),         # shorter than a chunk
     (5, 16, 1, 128, 128, 0.5),      # several short sequences per workgroup (suffix-like), odd count
     (5, 100, 1, 64, 128, None),     # several multi-chunk sequences per workgroup (the harness has 8 units), no initial state
+    (1, 150, 1, 192, 64, 0.3),      # 192-wide keys: three visits per chunk in the forward and dv passes
+    (1, 100, 2, 64, 192, 0.3),      # 192-wide values: three visits per chunk in the dq and dk passes
+    (1, 130, 1, 192, 192, None),    # both, no initial state
+    (1, 5, 130, 64, 64, 0.5),       # more than 128 heads
 ])
 def test_plain_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std):
     decays = oracle.head_decays(H)
@@ -54,6 +58,7 @@ def test_plain_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std):
     (1, 130, 1, 64, 64, 32),        # block divides chunk
     (1, 40, 1, 64, 64, 100),        # no full block at all
     (1, 130, 1, 256, 64, 32),       # widest contraction with block states written and their gradients read
+    (1, 130, 1, 192, 128, 48),      # three visits per chunk with block states
 ])
 def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
     decays = oracle.head_decays(H, (5, 12))
@@ -83,6 +88,8 @@ FUSED_NAMES = ("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0")
     (1, 2, 64, 100, 1, 128, 128, 0.5, 0),   # suffixes longer than a chunk: two parts
     (1, 1, 80, 130, 2, 64, 128, None, 30),  # ... three parts, tokens after the last boundary, no initial state
     (1, 1, 64, 128, 1, 64, 128, 0.3, 0),    # ... two full parts, dk != dv
+    (1, 2, 40, 9, 1, 192, 64, 0.5, 0),      # three visits per chunk in the forward and dv passes
+    (1, 2, 40, 9, 1, 128, 192, 0.5, 13),    # ... in the dq and dk passes, with trailing tokens
 ])
 def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std, tail):
     decays = oracle.head_decays(H, (4, 9))
@@ -102,6 +109,7 @@ def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std, ta
     (1, 1024, 1, 64, 128, None, 4),    # dk != dv, no initial state, 4 segments
     (1, 256, 1, 64, 64, 0.5, 1),       # too short to cut: same path as the plain entry point
     (1, 512, 1, 256, 64, 0.5, 2),      # 256-wide keys: the state-only walk visits every chunk twice
+    (1, 512, 1, 192, 64, 0.5, 2),      # 192-wide keys: three visits
 ])
 def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     decays = (0.97,) * H
@@ -188,7 +196,7 @@ def test_checkpoint_size_query(emu_lib, monkeypatch):
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 0
 
 
-@pytest.mark.parametrize("B,H,dk,dv", [(2, 3, 64, 128), (1, 2, 128, 64), (1, 1, 256, 256)])
+@pytest.mark.parametrize("B,H,dk,dv", [(2, 3, 64, 128), (1, 2, 128, 64), (1, 1, 256, 256), (1, 2, 192, 192), (2, 1, 64, 192)])
 def test_decode_step(emu_lib, B, H, dk, dv):
     """Three chained steps (no state, fresh buffer, in place) against the oracle's recurrent step."""
     decays = oracle.head_decays(H)

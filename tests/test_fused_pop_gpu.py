@@ -66,6 +66,7 @@ def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, ora
     (2, 8, 32, 1, 2, 64, 128),       # one-token suffixes
     (1, 3, 64, 16, 2, 256, 128),     # 256-wide keys: two visits per chunk in the forward and dv passes
     (1, 2, 96, 24, 2, 128, 256),     # 256-wide values: two visits per chunk in the dq and dk passes
+    (2, 3, 64, 16, 2, 192, 192),     # 192-wide keys and values: three visits per chunk in every pass
 ])
 def test_fused_parity_sweep(B, N, block, Ls, H, dk, dv):
     run_fused(B, N, block, Ls, H, dk, dv, 0.3, seed=N * block + Ls, decay_range=(5, 12))

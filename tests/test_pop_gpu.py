@@ -47,6 +47,7 @@ def run_pop(B, T, H, dk, dv, block, state_std, seed, decay_range=(5, 12), oracle
     (2, 256, 2, 128, 128, 64),     # block == chunk, headline head dims
     (1, 40, 2, 64, 64, 100),       # no full block: empty block_states
     (1, 192, 2, 128, 256, 64),
+    (2, 300, 2, 192, 64, 48),      # 192-wide keys: three visits per chunk, block states written and their gradients read
 ])
 def test_pop_parity_sweep(B, T, H, dk, dv, block):
     run_pop(B, T, H, dk, dv, block, 0.3, seed=T + block)

@@ -12,7 +12,7 @@ import oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-DIMS = (64, 128, 256)
+DIMS = (64, 128, 192, 256)
 
 
 def _decays(rng, H):

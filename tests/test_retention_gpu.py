@@ -57,7 +57,11 @@ def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, 
     (1, 300, 2, 128, 256, 0.02),     # config-3 head dims
     (1, 130, 2, 256, 128, 0.1),      # dk = 256
     (2, 2048, 4, 64, 128, 0.0),      # reference grads test shape (tests/test_fused_retention.py:240-282)
-    (1, 70, 128, 64, 64, 0.1),       # the largest supported head count (decays down to 1 - 2^-132, i.e. 1.0)
+    (1, 70, 128, 64, 64, 0.1),       # many heads (decays down to 1 - 2^-132, i.e. 1.0)
+    (1, 70, 512, 64, 64, 0.1),       # the largest supported head count
+    (2, 300, 4, 192, 128, 0.1),      # 192-wide keys: three visits per chunk in the forward and dv passes
+    (1, 200, 2, 64, 192, None),      # 192-wide values: three visits in the dq and dk passes
+    (2, 1000, 3, 192, 192, 0.05),    # both
     (4, 1000, 16, 128, 128, 0.1),    # the backward that carries dS once, one checkpoint and a ragged stretch after it
     (2, 513, 32, 128, 128, None),    # ... a one-token last chunk behind the only checkpoint, no state argument
     (1, 4100, 64, 128, 128, 0.05),   # ... eight checkpoints, 64 heads
