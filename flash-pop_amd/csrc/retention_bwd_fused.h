@@ -9,7 +9,17 @@
 //                         dS <- gamma^L dS + sum_j gamma^(j+1) q_j^T dO_j is done once and q, k, v,
 //                         dO are read once.
 //   "forward" workgroup   the dq pass (X = dO, W = v, Z = k, R = S^T), walking forward and
-//                         re-running the state recurrence from s0.
+//                         re-running the state recurrence from s0, or, with the states that the
+//                         forward pass left every few chunks, from those checkpoints: segment by
+//                         segment from the last to the first, close to the reverse workgroup of
+//                         its stream, so that rows read twice are read close together in time.
+//
+// With POP suffixes (the SFX instantiations) a suffix is one more stop of either walk at its block
+// boundary, with tensors of its own: it reads the state there and leaves it as it is.
+//
+// Outputs are stored, and q (which only the reverse workgroup reads) is loaded, with the
+// non-temporal hint: kept out of the caches they leave room for k, v and dO, which both workgroups
+// of a stream read.
 //
 // Both kinds keep the four (three) 64 x 128 input tiles of a chunk row-major in LDS, single
 // buffered; the next chunk waits in registers.  Operands that run along the features of a tile are
