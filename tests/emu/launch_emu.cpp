@@ -7,72 +7,31 @@
 #include "decode_step.h"
 #include "layer_ops.h"
 
-#include <thread>
 #include <vector>
 
 namespace fprt {
 thread_local LaneCtx g_lane;
 }
 
+#include "run_grid.h"
+
+// The pass kernel's instantiations are compiled one contraction width per translation unit
+// (pass_family.cpp, built once per width) so that the harness builds in parallel.
+int emu_pass_64(const fpk::PassArgs* planned, int n);
+int emu_pass_128(const fpk::PassArgs* planned, int n);
+int emu_pass_192(const fpk::PassArgs* planned, int n);
+int emu_pass_256(const fpk::PassArgs* planned, int n);
+
 namespace {
 
-template <typename Body>
-int run_grid(int nthreads, int nwg, int lds_bytes, Body body) {
-  // exactly the bytes the GPU launch reserves, on the heap so that ASan sees overruns
-  std::vector<char>* lds = new std::vector<char>(lds_bytes);
-  pthread_barrier_t wg_bar;
-  pthread_barrier_init(&wg_bar, nullptr, nthreads);
-  std::vector<fprt::WaveShared> waves(nthreads / 64);
-  for (auto& w : waves) pthread_barrier_init(&w.bar, nullptr, 64);
-  std::vector<std::thread> lanes;
-  for (int t = 0; t < nthreads; ++t) {
-    lanes.emplace_back([&, t] {
-      fprt::g_lane.tid = t;
-      fprt::g_lane.grid = nwg;
-      fprt::g_lane.wave = &waves[t >> 6];
-      fprt::g_lane.wg_bar = &wg_bar;
-      for (int wg = 0; wg < nwg; ++wg) {
-        fprt::g_lane.block = wg;
-        body(lds->data());
-        pthread_barrier_wait(&wg_bar);
-      }
-    });
+int run_family(const fpk::PassArgs* planned, int n) {
+  switch (planned[0].dA) {
+    case 64: return emu_pass_64(planned, n);
+    case 128: return emu_pass_128(planned, n);
+    case 192: return emu_pass_192(planned, n);
+    default: return emu_pass_256(planned, n);
   }
-  for (auto& th : lanes) th.join();
-  for (auto& w : waves) pthread_barrier_destroy(&w.bar);
-  pthread_barrier_destroy(&wg_bar);
-  delete lds;
-  return 0;
 }
-
-}  // namespace
-
-namespace {
-
-struct HarnessRun {
-  const fpk::PassArgs& a;
-  template <int DA, int MODE, int NH>
-  int go(int /*slot*/) const {
-    const int nwg = a.slots * a.H * (a.dB / fpk::BV);
-    return run_grid(fpk::NTHREADS_WS, nwg, fpk::lds_bytes_ws(DA), [&](char* l) {
-      fpk::retention_pass_ws<DA, MODE, NH>(a, fpk::tensors_of(a), l, fpk::place_workgroup(fprt::block_index(), nwg, 1).wg, nwg);
-    });
-  }
-};
-
-struct HarnessMultiRun {
-  const fpk::PassArgs* planned;
-  int n;
-  template <int DA, int MODE, int NH>
-  int go(int /*slot*/) const {
-    const fpk::PassArgs& a = planned[0];
-    const int nwg = a.slots * a.H * (a.dB / fpk::BV);
-    return run_grid(fpk::NTHREADS_WS, n * nwg, fpk::lds_bytes_ws(DA), [&](char* l) {
-      const fpk::WorkgroupId id = fpk::place_workgroup(fprt::block_index(), nwg, n);
-      fpk::retention_pass_ws<DA, MODE, NH>(a, fpk::tensors_of(planned[id.pass]), l, id.wg, nwg);
-    });
-  }
-};
 
 }  // namespace
 
@@ -82,7 +41,7 @@ int fpk_launch_pass(const fpk::PassArgs& args, void* /*stream*/, const char** er
     *err = why;
     return 1;
   }
-  return fpk::dispatch_pass(a, HarnessRun{a});
+  return run_family(&a, 1);
 }
 
 int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, const char** err) {
@@ -92,7 +51,7 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
     *err = why;
     return 1;
   }
-  return fpk::dispatch_pass(planned[0], HarnessMultiRun{planned, n});
+  return run_family(planned, n);
 }
 
 // the harness's stand-in for the library's own scratch array (host memory here)

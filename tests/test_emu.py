@@ -39,7 +39,6 @@ def _check_all(pairs):
     (1, 150, 1, 192, 64, 0.3),      # 192-wide keys: three visits per chunk in the forward and dv passes
     (1, 100, 2, 64, 192, 0.3),      # 192-wide values: three visits per chunk in the dq and dk passes
     (1, 130, 1, 192, 192, None),    # both, no initial state
-    (1, 5, 130, 64, 64, 0.5),       # more than 128 heads
 ])
 def test_plain_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std):
     decays = oracle.head_decays(H)
@@ -127,9 +126,9 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
 
 
 @pytest.mark.parametrize("B,nblk,block,Ls,H,state_std", [
-    (1, 4, 128, 16, 2, 0.5),     # two chunks per block
-    (2, 8, 64, 64, 1, None),     # block == chunk, suffixes as long as a chunk, no initial state
-    (1, 3, 192, 1, 2, 0.3),      # three chunks per block, one-token suffixes
+    (1, 4, 128, 16, 1, 0.5),     # two chunks per block
+    (1, 8, 64, 64, 1, None),     # block == chunk, suffixes as long as a chunk, no initial state
+    (1, 3, 192, 1, 1, 0.3),      # three chunks per block, one-token suffixes
 ])
 def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, block, Ls, H, state_std):
     """dk = dv = 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
@@ -152,11 +151,11 @@ def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, 
 
 
 @pytest.mark.parametrize("B,T,H,state_std,every", [
-    (1, 700, 2, 0.5, 128),      # ragged tail beyond the last checkpoint, initial state
+    (1, 700, 1, 0.5, 128),      # ragged tail beyond the last checkpoint, initial state
     (1, 512, 1, None, 256),     # the sequence ends on a checkpoint, no initial state
     (2, 520, 1, 0.3, 64),       # a checkpoint after every chunk, two sequences
     (1, 600, 1, 0.2, 1024),     # interval longer than the sequence: no checkpoint at all
-    (1, 576, 2, 0.4, 0),        # no checkpoint buffer: the fused backward walks forward from s0
+    (1, 576, 1, 0.4, 0),        # no checkpoint buffer: the fused backward walks forward from s0
 ])
 def test_fused_backward_with_checkpoints(emu_lib, monkeypatch, B, T, H, state_std, every):
     """dk = dv = 128 and at least eight chunks: the backward that carries dS once, beside the
@@ -196,7 +195,8 @@ def test_checkpoint_size_query(emu_lib, monkeypatch):
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 0
 
 
-@pytest.mark.parametrize("B,H,dk,dv", [(2, 3, 64, 128), (1, 2, 128, 64), (1, 1, 256, 256), (1, 2, 192, 192), (2, 1, 64, 192)])
+@pytest.mark.parametrize("B,H,dk,dv", [(2, 3, 64, 128), (1, 2, 128, 64), (1, 1, 256, 256), (1, 2, 192, 192), (2, 1, 64, 192),
+                                       (1, 130, 64, 64)])   # more than 128 heads
 def test_decode_step(emu_lib, B, H, dk, dv):
     """Three chained steps (no state, fresh buffer, in place) against the oracle's recurrent step."""
     decays = oracle.head_decays(H)

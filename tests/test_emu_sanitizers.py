@@ -7,16 +7,13 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 EMU = os.path.join(HERE, "emu")
-CSRC = os.path.join(HERE, "..", "flash-pop_amd", "csrc")
 
 
 def test_all_entry_points_under_asan_and_ubsan(tmp_path):
     exe = str(tmp_path / "asan_driver")
-    cxx = os.environ.get("EMU_CXX", "/opt/rocm/llvm/bin/clang++")
-    subprocess.run([cxx, "-std=c++17", "-O1", "-g", "-pthread", "-fsanitize=address,undefined",
-                    "-fno-sanitize-recover=all", "-fno-omit-frame-pointer", f"-I{EMU}", f"-I{CSRC}",
-                    os.path.join(EMU, "asan_driver.cpp"), os.path.join(EMU, "launch_emu.cpp"),
-                    os.path.join(CSRC, "flashpop_api.cpp"), "-o", exe], check=True)
+    build_env = dict(os.environ, EMU_OUT=exe, EMU_MAIN=os.path.join(EMU, "asan_driver.cpp"), EMU_OPT="-O1",
+                     EMU_FLAGS="-fsanitize=address,undefined -fno-sanitize-recover=all -fno-omit-frame-pointer")
+    subprocess.run([os.path.join(EMU, "build_emu.sh")], check=True, env=build_env)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
     res = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=1500)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-6000:]
