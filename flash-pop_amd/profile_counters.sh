@@ -23,6 +23,10 @@ CMD=$BENCH run fetch --pmc FETCH_SIZE
 CMD=$BENCH run write --pmc WRITE_SIZE
 CMD=$COPY run copy_fetch --pmc FETCH_SIZE
 CMD=$COPY run copy_write --pmc WRITE_SIZE
+# long context, few streams (benchmark configuration 3): the split-sequence passes
+LONG="python3 $R/bench.py --steps 8 --warmup 4 --no-cpu --no-pop --no-layer --no-model"
+CMD=$LONG run long_trace --kernel-trace --stats
+rm -f "$O/long_trace/r_kernel_trace.csv"
 # the model-level step of benchmark configuration 5 (12-layer harness around the ops): which kernels its time goes to
 MODEL="python3 $R/bench.py --steps 10 --warmup 2 --spin-up 0 --no-cpu --no-pop --no-long --no-layer"
 CMD=$MODEL run model_trace --kernel-trace --stats

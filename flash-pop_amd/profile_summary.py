@@ -123,6 +123,12 @@ def main():
         for l in lines:
             print(l)
 
+    if os.path.exists(p("long_trace", "r_kernel_stats.csv")):
+        print("\n## Long-context run (config 3: B2 H8 T16384 dk128 dv256): kernel trace\n")
+        print("| kernel | calls | average | min | max |\n|---|---|---|---|---|")
+        for name, calls, avg, lo, hi in kernel_stats(p("long_trace", "r_kernel_stats.csv")):
+            print(f"| {name} | {calls} | {avg:.1f} us | {lo:.1f} us | {hi:.1f} us |")
+
     if os.path.exists(p("model_trace", "r_kernel_stats.csv")):
         model_breakdown(p("model_trace", "r_kernel_stats.csv"))
 
