@@ -184,7 +184,10 @@ bool use_fused_backward(const Shape& s, const void* d_blocks) {
     if (std::strcmp(e, "passes") == 0) return false;
     if (std::strcmp(e, "fused") == 0) return true;
   }
-  return 4LL * s.B * s.H >= fpk_compute_units();
+  // two workgroups per stream: with fewer than two thirds of the compute units covered the column-tiled
+  // passes, which fill the chip, are faster (256 units, T = 4096: 64 streams 0.33 ms against 0.30 ms; with POP
+  // suffixes, 80 streams 0.375 against 0.353 ms)
+  return 3LL * s.B * s.H >= fpk_compute_units();
 }
 
 // Tokens between the states that fp_retention_fwd_ckpt leaves for the backward (0: none wanted).

@@ -119,7 +119,7 @@ def test_random_cases_for_the_backward_that_carries_ds_once():
     lib = _lib.load()
     for case in range(10):
         H = rng.choice([8, 16, 32])
-        B = 64 // H * rng.randint(1, 2)
+        B = 96 // H * rng.randint(1, 2)
         decays = _decays(rng, H)
         state_std = rng.choice([None, 0.2])
         if case % 2 == 0:

@@ -62,9 +62,9 @@ def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, 
     (2, 300, 4, 192, 128, 0.1),      # 192-wide keys: three visits per chunk in the forward and dv passes
     (1, 200, 2, 64, 192, None),      # 192-wide values: three visits in the dq and dk passes
     (2, 1000, 3, 192, 192, 0.05),    # both
-    (4, 1000, 16, 128, 128, 0.1),    # the backward that carries dS once, one checkpoint and a ragged stretch after it
-    (2, 513, 32, 128, 128, None),    # ... a one-token last chunk behind the only checkpoint, no state argument
-    (1, 4100, 64, 128, 128, 0.05),   # ... eight checkpoints, 64 heads
+    (6, 1000, 16, 128, 128, 0.1),    # the backward that carries dS once, one checkpoint and a ragged stretch after it
+    (3, 513, 32, 128, 128, None),    # ... a one-token last chunk behind the only checkpoint, no state argument
+    (2, 2100, 64, 128, 128, 0.05),   # ... four checkpoints, 64 heads
 ])
 def test_parity_sweep(B, T, H, dk, dv, state_std):
     run_plain(B, T, H, dk, dv, state_std, seed=T + dk)
@@ -106,7 +106,7 @@ def test_checkpointed_backward_against_oracle_and_plain_entry_points(hip_lib):
     (dk = dv = 128, enough streams): all results against the oracle; o, S, dk, dv and ds0 bit for bit
     those of the entry points without checkpoints (the checkpoints only serve dq)."""
     import ctypes
-    B, T, H = 4, 1600, 16
+    B, T, H = 6, 1600, 16
     decays = oracle.head_decays(H)
     q, k, v, s = (t.to(DEV) for t in hp.make_inputs(B, T, H, 128, 128, seed=11, state_std=0.3))
     d_o, d_s = (t.to(DEV) for t in hp.make_cotangents([(B, T, H, 128), (B, H, 128, 128)], seed=12))
