@@ -336,9 +336,20 @@ Shape segment_shape(const Shape& s, int segments) { return Shape{s.B * segments,
 // (backward walk over q, dO).
 int contributions(const Shape& seg, const double* decays, const void* w_rows, const void* z_rows, int reverse,
                   const Workspace& w, void* stream) {
+  const float sc = 1.0f / std::sqrt((float)seg.dk);
+  if (seg.dk == fpk::FB_D && seg.dv % fpk::FB_D == 0) {   // the kernel that holds 128 x 128 of the state per workgroup
+    fpk::ContribArgs c;
+    std::memset(&c, 0, sizeof c);
+    c.W = in(w_rows); c.Z = in(z_rows); c.U = w.contrib;
+    c.B = seg.B; c.T = seg.T; c.H = seg.H; c.dB = seg.dv; c.reverse = reverse;
+    c.s_update = reverse ? 1.f : sc;
+    for (int h = 0; h < seg.H; ++h) c.log2g[h] = (float)std::log2(decays[h]);
+    const char* msg = "";
+    if (fpk_launch_contrib(c, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "%s: %s", reverse ? "dS contributions" : "S contributions", msg);
+    return FP_OK;
+  }
   fpk::PassArgs a;
   fill_common(a, seg, decays);
-  const float sc = 1.0f / std::sqrt((float)seg.dk);
   a.X = in(w_rows);   // never read
   a.W = in(w_rows); a.Z = in(z_rows);
   a.Rout = w.contrib;

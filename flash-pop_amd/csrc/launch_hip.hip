@@ -4,6 +4,7 @@
 #include "device_rt.h"
 #include "pass_dispatch.h"
 #include "segment_scan.h"
+#include "segment_contrib.h"
 #include "retention_bwd_fused.h"
 #include "decode_step.h"
 #include "layer_ops.h"
@@ -46,6 +47,12 @@ __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const f
   fpk::segment_scan(args);
 }
 
+template <bool REV>
+__global__ __launch_bounds__(fpk::FB_THREADS) void segment_contrib_kernel(const fpk::ContribArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::segment_contrib<REV>(args, lds);
+}
+
 __global__ __launch_bounds__(fpk::DECODE_THREADS) void decode_step_kernel(const fpk::DecodeArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   fpk::decode_step(args, lds);
@@ -68,7 +75,7 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(cons
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
-static_assert(2 * fpk::PASS_KERNELS <= 61, "one bit per kernel instantiation, single and paired");
+static_assert(2 * fpk::PASS_KERNELS <= 59, "one bit per kernel instantiation, single and paired; the top four for the others");
 std::atomic<uint64_t> g_armed[kMaxDevices];
 
 template <typename Kernel, typename... More>
@@ -226,6 +233,41 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* stream, const char** 
     hipLaunchKernelGGL(retention_bwd_fused_pop_kernel, grid, threads, fpk::fb_lds_bytes(), static_cast<hipStream_t>(stream), a);
   else
     hipLaunchKernelGGL(retention_bwd_fused_kernel, grid, threads, fpk::fb_lds_bytes(), static_cast<hipStream_t>(stream), a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    *err = hipGetErrorString(e);
+    return 1;
+  }
+  return 0;
+}
+
+int fpk_launch_contrib(const fpk::ContribArgs& a, void* stream, const char** err) {
+  if (const char* why = fpk::check_contrib(a)) {
+    *err = why;
+    return 1;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    *err = "hipGetDevice failed";
+    return 1;
+  }
+  const void* const kernel = a.reverse ? reinterpret_cast<const void*>(segment_contrib_kernel<true>)
+                                       : reinterpret_cast<const void*>(segment_contrib_kernel<false>);
+  const uint64_t bit = 1ull << (a.reverse ? 60 : 61);
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & bit)) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, fpk::sc_lds_bytes()) != hipSuccess) {
+      (void)hipGetLastError();
+      *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
+      return 1;
+    }
+    if (tracked) g_armed[dev].fetch_or(bit, std::memory_order_release);
+  }
+  const dim3 grid((unsigned)(a.B * a.H * (a.dB / fpk::FB_D))), threads(fpk::FB_THREADS);
+  if (a.reverse)
+    hipLaunchKernelGGL(segment_contrib_kernel<true>, grid, threads, fpk::sc_lds_bytes(), static_cast<hipStream_t>(stream), a);
+  else
+    hipLaunchKernelGGL(segment_contrib_kernel<false>, grid, threads, fpk::sc_lds_bytes(), static_cast<hipStream_t>(stream), a);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     *err = hipGetErrorString(e);

@@ -92,6 +92,18 @@ struct ScanArgs {
   int B, S, H, M, Tseg, reverse;
   float log2g[MAX_HEADS];
 };
+// State-only pass for states of 128 rows (segment_contrib.h): U[b][h] = what sequence b adds to a
+// zero state, sum_j weight(j) W[j]^T Z[j] with weight(j) = s_update gamma^(T - 1 - j) walking forward
+// (`reverse` = 0) and s_update gamma^(j + 1) walking backward.  W [B,T,H,128], Z [B,T,H,dB],
+// U [B,H,128,dB], bf16; T a multiple of CH, dB a multiple of 128.
+struct ContribArgs {
+  const uint16_t* W;
+  const uint16_t* Z;
+  uint16_t* U;
+  int B, T, H, dB, reverse;
+  float s_update;
+  float log2g[MAX_HEADS];
+};
 // One recurrent (decode) step for every (batch, head):  S' = gamma S + (scale k)^T v,  o = q S'.
 // q, k [B,H,dk]; v, o [B,H,dv]; S [B,H,dk,dv]; all bf16, fp32 arithmetic.  s_out may be s_in.
 struct DecodeArgs {
@@ -191,6 +203,9 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);
+
+// Launches the state-only pass for states of 128 rows (B H dB / 128 workgroups).  Same conventions.
+int fpk_launch_contrib(const fpk::ContribArgs& args, void* stream, const char** err);
 
 // Bytes of the library's own scratch array (one per device, see fpk_static_scratch).
 namespace fpk {

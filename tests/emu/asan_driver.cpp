@@ -132,6 +132,7 @@ int main() {
   rc |= plain(1, 130, 1, 256, 64, false);     // two visits per chunk, state as stored
   rc |= plain(1, 100, 1, 192, 192, false);    // three visits per chunk
   rc |= plain(1, 512, 1, 64, 128, true);      // cut into segments (state-only walk, scan)
+  rc |= plain(1, 640, 1, 128, 256, true);     // ... with the state-only kernel for 128-wide keys, two workgroups per segment
   rc |= pop(1, 287, 1, 64, 128, 144);
   rc |= pop(2, 28, 1, 64, 64, 15);
   rc |= pop(1, 40, 1, 64, 64, 100);           // no full block

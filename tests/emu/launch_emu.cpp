@@ -3,6 +3,7 @@
 #include "device_rt.h"
 #include "pass_dispatch.h"
 #include "segment_scan.h"
+#include "segment_contrib.h"
 #include "retention_bwd_fused.h"
 #include "decode_step.h"
 #include "layer_ops.h"
@@ -73,6 +74,17 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* /*stream*/, const cha
   return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(), [&](char* l) {
     if (a.block > 0) fpk::fused_bwd<true>(a, l, fprt::block_index());
     else fpk::fused_bwd<false>(a, l, fprt::block_index());
+  });
+}
+
+int fpk_launch_contrib(const fpk::ContribArgs& a, void* /*stream*/, const char** err) {
+  if (const char* why = fpk::check_contrib(a)) {
+    *err = why;
+    return 1;
+  }
+  return run_grid(fpk::FB_THREADS, a.B * a.H * (a.dB / fpk::FB_D), fpk::sc_lds_bytes(), [&](char* l) {
+    if (a.reverse) fpk::segment_contrib<true>(a, l);
+    else fpk::segment_contrib<false>(a, l);
   });
 }
 

@@ -109,6 +109,8 @@ def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std, ta
     (1, 256, 1, 64, 64, 0.5, 1),       # too short to cut: same path as the plain entry point
     (1, 512, 1, 256, 64, 0.5, 2),      # 256-wide keys: the state-only walk visits every chunk twice
     (1, 512, 1, 192, 64, 0.5, 2),      # 192-wide keys: three visits
+    (1, 640, 1, 128, 128, 0.5, 2),     # 128-wide keys: the state-only kernel with the whole state tile per workgroup, 5 chunks
+    (1, 1024, 1, 128, 256, None, 4),   # ... two workgroups per sequence (256-wide values), 4 chunks per segment
 ])
 def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     decays = (0.97,) * H
