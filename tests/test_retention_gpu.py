@@ -295,10 +295,11 @@ def test_decode_step_kernel_256_steps():
     hp.assert_close(s1, s1_ref, "state, no state")
 
 
-@pytest.mark.parametrize("B,T,H,dk,dv", [(1, 8192, 2, 128, 128), (1, 4096, 2, 256, 128)])
+@pytest.mark.parametrize("B,T,H,dk,dv", [(1, 8192, 2, 128, 128), (1, 4096, 2, 256, 128), (2, 2240, 3, 128, 256)])
 def test_split_entry_points_long_sequence_few_streams(B, T, H, dk, dv):
     """fp_retention_*_split on shapes the library cuts into segments (a few streams on a 256-CU device; with
-    256-wide keys the state-only walk visits every chunk twice): against the oracle, against the unsplit
+    256-wide keys the state-only walk visits every chunk twice; the last case has 7 segments of 5 chunks and two
+    workgroups per segment in the state-only kernel for 128-wide keys): against the oracle, against the unsplit
     entry points, and the workspace argument checks."""
     from flash_pop_amd import _lib
     lib = _lib.load()
