@@ -34,13 +34,24 @@ __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_multi_kernel(
 
 __global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_kernel(const fpk::FusedBwdArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::fused_bwd<false>(args, lds, fprt::block_index());
+  fpk::fused_bwd<fpk::FB_PLAIN>(args, lds, fprt::block_index());
 }
 
-// the same with POP suffixes at the block boundaries
+// the same with POP suffixes at the block boundaries, as extra stops of the walks
 __global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_pop_kernel(const fpk::FusedBwdArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::fused_bwd<true>(args, lds, fprt::block_index());
+  fpk::fused_bwd<fpk::FB_STOPS>(args, lds, fprt::block_index());
+}
+
+// ... with suffixes of at most 16 tokens folded into the chunks at their boundaries, and the kernel for what stays
+// inside such a suffix
+__global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_fold_kernel(const fpk::FusedBwdArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::fused_bwd<fpk::FB_FOLD>(args, lds, fprt::block_index());
+}
+__global__ __launch_bounds__(fpk::SI_THREADS) void suffix_intra_bwd_kernel(const fpk::FusedBwdArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::suffix_intra_bwd(args, lds);
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -75,7 +86,7 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(cons
 // no thread calls hipFuncSetAttribute for it again (which matters to callers that capture
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
-static_assert(2 * fpk::PASS_KERNELS <= 59, "one bit per kernel instantiation, single and paired; the top four for the others");
+static_assert(2 * fpk::PASS_KERNELS <= 57, "one bit per kernel instantiation, single and paired; the top six for the others");
 std::atomic<uint64_t> g_armed[kMaxDevices];
 
 template <typename Kernel, typename... More>
@@ -204,41 +215,68 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
   return fpk::dispatch_pass(planned[0], DeviceMultiRun{planned, n, static_cast<hipStream_t>(stream), err});
 }
 
-int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* stream, const char** err) {
-  if (const char* why = fpk::check_fused_bwd(a)) {
-    *err = why;
-    return 1;
-  }
+namespace {
+
+// opts a kernel into `lds` bytes of dynamic LDS once per device (bit `bit` of the per-device word)
+int arm(const void* kernel, int lds, int bit, const char** err) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     *err = "hipGetDevice failed";
     return 1;
   }
-  const bool pop = a.block > 0;
-  const void* const kernel = pop ? reinterpret_cast<const void*>(retention_bwd_fused_pop_kernel)
-                                 : reinterpret_cast<const void*>(retention_bwd_fused_kernel);
-  // the opt-in to more than 64 KB of LDS, once per device (the top bits of the per-device word)
-  const uint64_t bit = 1ull << (pop ? 62 : 63);
+  const uint64_t mask = 1ull << bit;
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & bit)) {
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, fpk::fb_lds_bytes()) != hipSuccess) {
+  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & mask)) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(bit, std::memory_order_release);
+    if (tracked) g_armed[dev].fetch_or(mask, std::memory_order_release);
   }
-  const dim3 grid((unsigned)(2 * a.B * a.H)), threads(fpk::FB_THREADS);
-  if (pop)
-    hipLaunchKernelGGL(retention_bwd_fused_pop_kernel, grid, threads, fpk::fb_lds_bytes(), static_cast<hipStream_t>(stream), a);
-  else
-    hipLaunchKernelGGL(retention_bwd_fused_kernel, grid, threads, fpk::fb_lds_bytes(), static_cast<hipStream_t>(stream), a);
+  return 0;
+}
+
+int launched(const char** err) {
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     *err = hipGetErrorString(e);
     return 1;
   }
   return 0;
+}
+
+}  // namespace
+
+int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char** err) {
+  fpk::FusedBwdArgs a = args;
+  a.fold = a.block > 0 && a.Ls <= fpk::FB_SFX_ROWS;
+  if (const char* why = fpk::check_fused_bwd(a)) {
+    *err = why;
+    return 1;
+  }
+  const hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)(2 * a.B * a.H)), threads(fpk::FB_THREADS);
+  if (a.fold) {
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_fold_kernel), fpk::fb_fold_lds_bytes(), 59, err)) return 1;
+    if (arm(reinterpret_cast<const void*>(suffix_intra_bwd_kernel), fpk::si_lds_bytes(), 58, err)) return 1;
+    hipLaunchKernelGGL(retention_bwd_fused_fold_kernel, grid, threads, fpk::fb_fold_lds_bytes(), st, a);
+    if (launched(err)) return 1;
+    // what stays inside the suffixes, after the part of dq_s that comes from the carried state is written
+    const long long pairs = (long long)a.B * (a.T / a.block + 1) * a.H;
+    const long long wgs = 8LL * fpk_compute_units();
+    hipLaunchKernelGGL(suffix_intra_bwd_kernel, dim3((unsigned)(pairs < wgs ? pairs : wgs)), dim3(fpk::SI_THREADS),
+                       fpk::si_lds_bytes(), st, a);
+    return launched(err);
+  }
+  if (a.block > 0) {
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_pop_kernel), fpk::fb_lds_bytes(), 62, err)) return 1;
+    hipLaunchKernelGGL(retention_bwd_fused_pop_kernel, grid, threads, fpk::fb_lds_bytes(), st, a);
+  } else {
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel), fpk::fb_lds_bytes(), 63, err)) return 1;
+    hipLaunchKernelGGL(retention_bwd_fused_kernel, grid, threads, fpk::fb_lds_bytes(), st, a);
+  }
+  return launched(err);
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* stream, const char** err) {
@@ -312,19 +350,6 @@ int fpk_launch_decode(const fpk::DecodeArgs& a, void* stream, const char** err) 
   }
   return 0;
 }
-
-namespace {
-
-int launched(const char** err) {
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    *err = hipGetErrorString(e);
-    return 1;
-  }
-  return 0;
-}
-
-}  // namespace
 
 int fpk_launch_rotary(const fpk::RotaryArgs& args, void* stream, const char** err) {
   fpk::RotaryArgs a = args;

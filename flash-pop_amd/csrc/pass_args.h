@@ -140,6 +140,7 @@ struct FusedBwdArgs {
   const uint16_t *q_sfx, *k_sfx, *v_sfx, *dO_sfx;
   uint16_t *dq_sfx, *dk_sfx, *dv_sfx;
   int block, Ls;
+  int fold;                                // suffixes of at most 16 tokens: folded into the chunks at their boundaries (FB_FOLD), set by the launcher
   int B, T, H;
   float scale;                             // dk^-1/2
   float log2g[MAX_HEADS];

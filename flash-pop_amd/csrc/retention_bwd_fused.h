@@ -52,6 +52,20 @@ constexpr int FB_TILE = CH * FB_LD;        // elements of a 64 x 128 tile
 constexpr int FB_XP = 32 * 32;             // elements of one score tile in operand layout
 // reverse workgroup: q, k, v, dO tiles; bf16 copy of dS; two staging tiles; six score tiles
 constexpr int fb_lds_bytes() { return 2 * (4 * FB_TILE + FB_D * FB_LD + 2 * FB_TILE + 6 * FB_XP); }
+// How POP suffixes take part in the walks:
+//   FB_PLAIN  none
+//   FB_STOPS  a suffix is one more stop of either walk (Ls <= 64)
+//   FB_FOLD   suffixes of at most 16 tokens: only what couples a suffix to the carried states is done here, as part of
+//             the chunk that starts at its boundary (the reverse workgroup adds sum_j gamma^(j+1) q_s[j]^T dO_s[j] to
+//             dS as one more k-step of that chunk's update, the forward workgroup reads the state out for dO_s beside
+//             the chunk's own read-out and writes that part of dq_s); what stays inside a suffix (dk_s, dv_s and the
+//             rest of dq_s) is the work of suffix_intra_bwd, which runs afterwards.  Both walks take one more, empty,
+//             chunk at T for the suffix there.
+enum FbMode { FB_PLAIN = 0, FB_STOPS = 1, FB_FOLD = 2 };
+constexpr int FB_SFX_ROWS = 16;                         // longest suffix of FB_FOLD
+constexpr int FB_SFX_TILE = 2 * FB_SFX_ROWS * FB_LD;    // elements of a 32 x 128 tile (the read-out wants 32 rows)
+// FB_FOLD: the reverse workgroup adds the first 16 rows of q_s and dO_s, the forward one a dO_s tile and two staging tiles
+constexpr int fb_fold_lds_bytes() { return fb_lds_bytes() + 2 * FB_SFX_TILE; }
 
 namespace fb {
 
@@ -358,14 +372,17 @@ FP_DEVICE void score_weights(float s_intra, float lg, bool diagonal, bool revers
 // SFX: POP suffixes hang off the block boundaries (item_backward).  Nothing downstream of a suffix
 // reaches back into it, so it reads no dS (no read-out), and what it adds to dS, the gradient of
 // the state it read, is not decayed.
-template <int PASS, bool SFX>
+template <int PASS, int MODE>
 FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   using namespace fb;
+  constexpr bool SFX = MODE == FB_STOPS, FOLD = MODE == FB_FOLD;
   const Common k = make_common(p, stream);
   uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // tiles: 0 q, 1 dO, 2 k, 3 v
   uint16_t* const Rt = TL + 4 * FB_TILE;                   // bf16(dS) as Rt[n = dv][a = dk]
   uint16_t* const OUT = Rt + FB_D * FB_LD;                 // staging: 0 dv, 1 dk
   uint16_t* const XP = OUT + 2 * FB_TILE;                  // score tiles [pass][tile][k-step][lane]
+  uint16_t* const QS = XP + 6 * FB_XP;                     // FOLD: 16 rows of q_s, then 16 rows of dO_s
+  uint16_t* const GS = QS + FB_SFX_ROWS * FB_LD;
   const uint16_t *Qs = TL, *Gs = TL + FB_TILE, *Ks = TL + 2 * FB_TILE, *Vs = TL + 3 * FB_TILE;
 
   constexpr int pass = PASS;
@@ -399,14 +416,30 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
 
   const Sources<2> src_qg = {{p.q, p.dO}, {p.q_sfx, p.dO_sfx}};   // q: read by this workgroup only
   const Sources<2> src_kv = {{p.k, p.v}, {p.k_sfx, p.v_sfx}};
-  const int nitems = item_count(k);
-  Item cur = item_backward(k, 0), nxt = item_backward(k, 1), prev = cur;
-  u32x4 pf_qg[4], pf_kv[4];
+  // FOLD: the chunks from the one past the end (empty; it carries the suffix at T) down to the first
+  auto item_of = [&](int it) { return FOLD ? chunk_item(k, k.nch - it) : item_backward(k, it); };
+  const int nitems = FOLD ? k.nch + 1 : item_count(k);
+  // FOLD: the suffix that hangs off the first token of the chunk visited it-th (L = 0: none), and this thread's
+  // 16 bytes of its q_s (threads 0..255) or dO_s rows
+  auto suffix_of = [&](int it) {
+    const int t0 = (k.nch - it) * CH;
+    return it >= 0 && it < nitems && t0 % k.block == 0 ? suffix_item(k, t0 / k.block) : Item{0u, 0, false};
+  };
+  auto load_suffix = [&](int it) {
+    const Item sx = suffix_of(it);
+    const fprt::BufView v = item_view(k, nullptr, k.tid < 256 ? (const void*)p.q_sfx : (const void*)p.dO_sfx, Item{sx.row, sx.L, true});
+    return fprt::buf_load128(v, (uint32_t)((k.tid & 255) >> 4) * k.rowp + k.ld_piece * 16);
+  };
+  auto stage_suffix = [&](u32x4 v) { st128((k.tid < 256 ? QS : GS) + at((k.tid & 255) >> 4, 8 * k.ld_piece), v); };
+  Item cur = item_of(0), nxt = item_of(1), prev = cur;
+  u32x4 pf_qg[4], pf_kv[4], pf_s = {0, 0, 0, 0};
   load_tiles<2, 1>(k, src_qg, cur, pf_qg);
   load_tiles<2>(k, src_kv, cur, pf_kv);
+  if constexpr (FOLD) pf_s = load_suffix(0);
   load_state(k, Rt, p.ds_out ? p.ds_out + (size_t)stream * FB_D * FB_D : nullptr, false);
   stage_tiles<2>(k, TL, pf_qg);
   stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
+  if constexpr (FOLD) stage_suffix(pf_s);
   load_tiles<2, 1>(k, src_qg, nxt, pf_qg);
   load_tiles<2>(k, src_kv, nxt, pf_kv);
   fprt::block_sync();
@@ -424,7 +457,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     // a suffix of at most 16 tokens lives in the first k-step of tokens and the first 32-token half:
     // one score tile, one product each for the outputs and the state
     const bool brief = sfx && L <= 16;
-    const Item after = item_backward(k, it + 2);
+    const Item after = item_of(it + 2);
     // ---- the previous item's outputs leave (nothing writes the staging tiles before the next barrier)
     if (it > 0) {
       drain_tile(k, OUT, p.dv, p.dv_sfx, prev);
@@ -496,6 +529,8 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     }
     fprt::block_sync();
 
+    // FOLD: the next chunk's suffix rows travel during this stretch only (registers are scarce in the first one)
+    if constexpr (FOLD) pf_s = load_suffix(it + 1);
     // ---- stretch 2: Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]
     if (brief) {
       const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * rt), pq = ld128(xp_pass + lane * 8);
@@ -560,6 +595,17 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       }
     }
     }
+    if constexpr (FOLD) {
+      // the suffix at this chunk's first token: what it adds to dS is not decayed (it reads the state as it is there)
+      if (suffix_of(it).L > 0) {
+        const u32x4 ua = frag_rows(QS, tr_nat, 0, 32 * at_);
+        const u32x4 ub0 = frag_rows(GS, tr_nat, 0, 32 * nt0), ub1 = frag_rows(GS, tr_nat, 0, 32 * (nt0 + 1));
+        fprt::sched_fence();
+        const u32x4 wa = weigh(ua, wk0);
+        racc[0] = fprt::mfma_32x32x16_bf16(wa, ub0, racc[0]);
+        racc[1] = fprt::mfma_32x32x16_bf16(wa, ub1, racc[1]);
+      }
+    }
     // nobody reads this chunk's k and v tiles or the old copy of dS any more
     stage_tiles<2>(k, TL + 2 * FB_TILE, pf_kv);
     load_tiles<2>(k, src_kv, after, pf_kv);
@@ -570,6 +616,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     // ---- stretch 3: every read of this chunk's q and dO tiles is done
     stage_tiles<2>(k, TL, pf_qg);
     load_tiles<2, 1>(k, src_qg, after, pf_qg);
+    if constexpr (FOLD) stage_suffix(pf_s);
     fprt::block_sync();
     prev = cur;
     cur = nxt;
@@ -587,14 +634,17 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
 // STATE: the copy that waves 4..7 run; the two copies meet at the same barriers.
 // SFX: POP suffixes hang off the block boundaries (item_forward): a suffix reads R without
 // advancing it (no checkpoints in this form).
-template <bool STATE, bool SFX>
+template <bool STATE, int MODE>
 FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
   using namespace fb;
+  constexpr bool SFX = MODE == FB_STOPS, FOLD = MODE == FB_FOLD;
   const Common k = make_common(p, stream);
   uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // tiles: 0 X = dO, 1 W = v, 2 Z = k
   uint16_t* const Rt = TL + 3 * FB_TILE;                   // bf16(R) as Rt[n][a]
   uint16_t* const OUT = Rt + FB_D * FB_LD;
   uint16_t* const XP = OUT + FB_TILE;                      // score tiles (0,0), (0,1), (1,1)
+  uint16_t* const XS = XP + 3 * FB_XP;                     // FOLD: 32 rows for dO_s (the first Ls are not zero)
+  uint16_t* const OUTS = XS + FB_SFX_TILE;                 // FOLD: two staging tiles of 32 rows, used in turn
   const uint16_t *Xs = TL, *Ws = TL + FB_TILE, *Zs = TL + 2 * FB_TILE;
   const int g = k.g, c = k.c, lane = k.lane;
   constexpr bool state_role = STATE;
@@ -629,18 +679,37 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     return p.ckpt + (((size_t)k.b * nck + (seg - 1)) * p.H + k.h) * FB_D * FB_D;
   };
   // item visited in iteration `it`
-  auto item_of = [&](int it) { return SFX ? item_forward(k, it) : chunk_item(k, chunk_of(it)); };
-  const int nitems = SFX ? item_count(k) : k.nch;
+  // FOLD: the chunks in order and one more, empty, at T for the suffix there
+  auto item_of = [&](int it) { return SFX ? item_forward(k, it) : FOLD ? chunk_item(k, it) : chunk_item(k, chunk_of(it)); };
+  const int nitems = SFX ? item_count(k) : FOLD ? k.nch + 1 : k.nch;
+  // FOLD: the suffix that hangs off the first token of the chunk visited it-th (L = 0: none), this thread's 16 bytes
+  // of its dO_s rows (32 rows, zero from row Ls on), and its rows of dq_s
+  auto suffix_of = [&](int it) {
+    return it >= 0 && it < nitems && (it * CH) % k.block == 0 ? suffix_item(k, it * CH / k.block) : Item{0u, 0, false};
+  };
+  auto load_suffix = [&](int it) {
+    const Item sx = suffix_of(it);
+    return fprt::buf_load128(item_view(k, nullptr, p.dO_sfx, Item{sx.row, sx.L, true}), (uint32_t)k.ld_row * k.rowp + k.ld_piece * 16);
+  };
+  auto drain_suffix = [&](int it) {
+    const Item sx = suffix_of(it);
+    if (sx.L == 0) return;
+    const uint16_t* const tile = OUTS + ((it * CH / k.block) & 1) * FB_SFX_TILE;
+    fprt::buf_store128_nt(item_view(k, nullptr, p.dq_sfx, sx), (uint32_t)k.ld_row * k.rowp + k.ld_piece * 16,
+                          ld128(tile + at(k.ld_row, 8 * k.ld_piece)));
+  };
   const Sources<1> src_x = {{p.dO}, {p.dO_sfx}};
   const Sources<2> src_wz = {{p.v, p.k}, {p.v_sfx, p.k_sfx}};
   Item cur = item_of(0), nxt = item_of(1), prev = cur;
-  u32x4 pf_x[2], pf_wz[4];
+  u32x4 pf_x[2], pf_wz[4], pf_s = {0, 0, 0, 0};
   load_tiles<1>(k, src_x, cur, pf_x);
   load_tiles<2>(k, src_wz, cur, pf_wz);
+  if constexpr (FOLD) pf_s = load_suffix(0);
   // R[a][n] = S[n][a]: element (a, n) at n * 128 + a of a state matrix
   load_state(k, Rt, segment_state(nseg - 1), true);
   stage_tiles<1>(k, TL, pf_x);
   stage_tiles<2>(k, TL + FB_TILE, pf_wz);
+  if constexpr (FOLD) st128(XS + at(k.ld_row, 8 * k.ld_piece), pf_s);
   load_tiles<1>(k, src_x, nxt, pf_x);
   load_tiles<2>(k, src_wz, nxt, pf_wz);
   fprt::block_sync();
@@ -671,7 +740,10 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     const int L = cur.L;
     const bool brief = sfx && L <= 16;   // as in the reverse workgroup: first k-step of tokens, first half only
     const Item after = item_of(it + 2);
-    if (it > 0) drain_tile(k, OUT, p.dq, p.dq_sfx, prev);   // nothing writes the staging tile before the next barrier
+    if (it > 0) {   // nothing writes the staging tile before the next barrier
+      drain_tile(k, OUT, p.dq, p.dq_sfx, prev);
+      if constexpr (FOLD) drain_suffix(it - 1);
+    }
     f32x16 acc[2];
     if constexpr (state_role) {
       if (rt < 3 && !(brief && rt != 0)) {
@@ -727,9 +799,31 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
         acc[1][r] *= wread1;
       }
       }
+      if constexpr (FOLD) {
+        // the suffix at this chunk's first token reads the same R: its rows of dq_s, as far as they come from the state
+        const Item sx = suffix_of(it);
+        if (sx.L > 0) {
+          const uint16_t* const xsrow = XS + at(c, 8 * g);
+          f32x16 as = {0};
+          u32x4 ra[8], xs[8];
+#pragma unroll
+          for (int t = 0; t < 8; ++t) {
+            ra[t] = frag_cols(rrow, t);
+            xs[t] = frag_cols(xsrow, t);
+          }
+          fprt::sched_fence();
+#pragma unroll
+          for (int t = 0; t < 8; ++t) as = fprt::mfma_32x32x16_bf16(ra[t], xs[t], as);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) as[r] *= wread0;
+          put_output(OUTS + ((it * CH / k.block) & 1) * FB_SFX_TILE, c, 32 * rt, g, as);
+        }
+      }
     }
     fprt::block_sync();
 
+    // FOLD: the next chunk's suffix rows travel during the second stretch only (registers are scarce in the first)
+    if constexpr (FOLD) pf_s = load_suffix(it + 1);
     if constexpr (!state_role) {
       // Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]; tokens j < 32 reach both halves (tiles (0,0), (0,1)),
       // the others only the second
@@ -810,6 +904,7 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
 
     stage_tiles<2>(k, TL + FB_TILE, pf_wz);
     load_tiles<2>(k, src_wz, after, pf_wz);
+    if constexpr (FOLD) st128(XS + at(k.ld_row, 8 * k.ld_piece), pf_s);   // read in the first stretch only
     if constexpr (state_role) {
       if (fresh) {
 #pragma unroll
@@ -822,19 +917,123 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     nxt = after;
   }
   drain_tile(k, OUT, p.dq, p.dq_sfx, prev);
+  if constexpr (FOLD) drain_suffix(nitems - 1);
 }
 
 // launch index -> kind and stream: the reverse workgroups (the longer ones) come first
-// SFX: the form with POP suffixes (p.block > 0)
-template <bool SFX>
+// MODE: how POP suffixes take part (FbMode; p.block > 0 unless FB_PLAIN)
+template <int MODE>
 FP_DEVICE void fused_bwd(const FusedBwdArgs& p, char* lds, int block) {
   const int streams = p.B * p.H;
   if (block < streams) {
-    if (fprt::thread_index() < 256) fused_bwd_reverse<0, SFX>(p, lds, block);
-    else fused_bwd_reverse<1, SFX>(p, lds, block);
+    if (fprt::thread_index() < 256) fused_bwd_reverse<0, MODE>(p, lds, block);
+    else fused_bwd_reverse<1, MODE>(p, lds, block);
   }
-  else if (fprt::thread_index() < 256) fused_bwd_forward<false, SFX>(p, lds, block - streams);
-  else fused_bwd_forward<true, SFX>(p, lds, block - streams);
+  else if (fprt::thread_index() < 256) fused_bwd_forward<false, MODE>(p, lds, block - streams);
+  else fused_bwd_forward<true, MODE>(p, lds, block - streams);
+}
+
+// ---------------------------------------------------------------------------------------------
+// FB_FOLD, second launch: what stays inside a POP suffix of at most 16 tokens.  With
+// D[i][j] = scale gamma^(i - j) for j <= i, A = D . (q_s k_s^T) and dA = D . (dO_s v_s^T), both rounded to bf16:
+//   dv_s = A^T dO_s,   dk_s = dA^T q_s,   dq_s += dA k_s   (dq_s holds the part that came from the carried state).
+// One workgroup of 4 waves takes the (suffix, head) pairs m = block, block + grid, ...: three score tiles by one wave
+// each, then every wave a 32-column slice of each of the three outputs; the next pair's rows are on their way in
+// registers meanwhile.  The three products are the dv pass, the dk pass and the dq pass of the chunk kernels above
+// on one 16-token tile, and are written with their pieces.
+constexpr int SI_THREADS = 256;
+constexpr int si_lds_bytes() { return 2 * (7 * FB_SFX_TILE + 3 * FB_XP); }   // q, k, v, dO; dv, dk, dq; score tiles
+
+FP_DEVICE void suffix_intra_bwd(const FusedBwdArgs& p, char* lds) {
+  using namespace fb;
+  const int tid = fprt::thread_index(), wave = tid >> 6, lane = tid & 63, g = lane >> 5, c = lane & 31;
+  uint16_t* const TL = reinterpret_cast<uint16_t*>(lds);   // 0 q, 1 k, 2 v, 3 dO: 32 rows each, zero from row Ls on
+  uint16_t* const OUT = TL + 4 * FB_SFX_TILE;              // 0 dv, 1 dk, 2 dq
+  uint16_t* const XP = OUT + 3 * FB_SFX_TILE;
+  const uint32_t rowp = (uint32_t)p.H * FB_D * 2;
+  const int pairs = p.B * (p.T / p.block + 1) * p.H;
+  const int ld_row = tid >> 4, ld_piece = tid & 15;        // this thread's 16-byte pieces: rows ld_row and ld_row + 16
+  const TrLane tr_acc = tr_lane(lane, TR_ACC);
+  // pass of the score tile this wave makes (waves 0..2): X, W and whether it is the backward-walking kind
+  //   0 dv: X = k, W = q, reverse     1 dk: X = v, W = dO, reverse     2 dq: X = dO, W = v, forward
+  const int xt = wave == 0 ? 1 : wave == 1 ? 2 : 3, wt = wave == 0 ? 0 : wave == 1 ? 3 : 2;
+  const uint16_t* const s_xrow = TL + xt * FB_SFX_TILE + at(c, 8 * g);
+  const uint16_t* const s_wrow = TL + wt * FB_SFX_TILE + at(score_row(c), 8 * g);
+
+  auto view = [&](const void* base, int m, int rows) {
+    const char* ptr = static_cast<const char*>(base) + ((size_t)(m / p.H) * p.Ls * p.H + (size_t)(m % p.H)) * FB_D * 2;
+    return fprt::make_buf(ptr, rows > 0 ? (uint32_t)(rows - 1) * rowp + FB_D * 2 : 0u);
+  };
+  // registers <- the rows of pair m: q, k, v, dO (two pieces each) and the dq_s written so far (one piece)
+  struct Rows {
+    u32x4 in[8], dq;
+  };
+  auto load = [&](int m, Rows& r) {
+    const int rows = m < pairs ? p.Ls : 0, mm = m < pairs ? m : 0;
+    const void* const src[4] = {p.q_sfx, p.k_sfx, p.v_sfx, p.dO_sfx};
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const fprt::BufView v = view(src[x], mm, rows);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) r.in[2 * x + u] = fprt::buf_load128(v, (uint32_t)(ld_row + 16 * u) * rowp + ld_piece * 16);
+    }
+    r.dq = fprt::buf_load128(view(p.dq_sfx, mm, rows), (uint32_t)ld_row * rowp + ld_piece * 16);
+  };
+
+  Rows cur;
+  load(fprt::block_index(), cur);
+  for (int m = fprt::block_index(); m < pairs; m += fprt::grid_size()) {
+    const float lg = p.log2g[m % p.H];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) st128(TL + x * FB_SFX_TILE + at(ld_row + 16 * u, 8 * ld_piece), cur.in[2 * x + u]);
+    }
+    const u32x4 dq_state = cur.dq;
+    load(m + fprt::grid_size(), cur);
+    fprt::block_sync();
+    if (wave < 3) {
+      float mw[16];
+      score_weights(p.scale, lg, true, wave < 2, c, g, mw);
+      u32x4 wf[8], xf[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        wf[t] = frag_cols(s_wrow, t);
+        xf[t] = frag_cols(s_xrow, t);
+      }
+      fprt::sched_fence();
+      f32x16 sc = {0};
+#pragma unroll
+      for (int t = 0; t < 8; ++t) sc = fprt::mfma_32x32x16_bf16(wf[t], xf[t], sc);
+      score_finish(sc, mw, true, wave < 2, c, g, XP + wave * FB_XP, lane);
+    }
+    fprt::block_sync();
+    // Y^T[n][i] = sum_j Z^T[n][j] P^T[j][i] for this wave's 32 columns n of each output: Z = dO, q, k
+#pragma unroll
+    for (int o = 0; o < 3; ++o) {
+      const uint16_t* const Zs = TL + (o == 0 ? 3 : o == 1 ? 0 : 1) * FB_SFX_TILE;
+      const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * wave), pq = ld128(XP + o * FB_XP + lane * 8);
+      f32x16 acc = {0};
+      acc = fprt::mfma_32x32x16_bf16(za, pq, acc);
+      put_output(OUT + o * FB_SFX_TILE, c, 32 * wave, g, acc);
+    }
+    fprt::block_sync();
+    // rows < Ls leave; dq_s is the sum with what the carried state gave
+    {
+      const u32x4 dvv = ld128(OUT + at(ld_row, 8 * ld_piece)), dkv = ld128(OUT + FB_SFX_TILE + at(ld_row, 8 * ld_piece));
+      const u32x4 dqi = ld128(OUT + 2 * FB_SFX_TILE + at(ld_row, 8 * ld_piece));
+      u32x4 dqv;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        dqv[d] = fprt::pack_bf16x2(bf16_elem(dqi, 2 * d) + bf16_elem(dq_state, 2 * d), bf16_elem(dqi, 2 * d + 1) + bf16_elem(dq_state, 2 * d + 1));
+      const uint32_t off = (uint32_t)ld_row * rowp + ld_piece * 16;
+      fprt::buf_store128_nt(view(p.dv_sfx, m, p.Ls), off, dvv);
+      fprt::buf_store128_nt(view(p.dk_sfx, m, p.Ls), off, dkv);
+      fprt::buf_store128_nt(view(p.dq_sfx, m, p.Ls), off, dqv);
+    }
+    // (the next pair's rows overwrite the input tiles only after the barrier that follows its staging... they are
+    // staged before it: every read of the input tiles is behind the barrier above)
+  }
 }
 
 // What the kernel assumes about its arguments; nullptr or a message for the caller.
@@ -847,6 +1046,7 @@ inline const char* check_fused_bwd(const FusedBwdArgs& a) {
   if (a.block > 0) {
     if (a.block % CH != 0 || a.T % a.block != 0 || a.Ls < 1 || a.Ls > CH)
       return "fused backward with suffixes: block a multiple of 64 that divides T, 1 <= Ls <= 64";
+    if (a.fold && a.Ls > FB_SFX_ROWS) return "fused backward with folded suffixes: Ls <= 16";
     if (!a.q_sfx || !a.k_sfx || !a.v_sfx || !a.dO_sfx || !a.dq_sfx || !a.dk_sfx || !a.dv_sfx)
       return "fused backward with suffixes: all seven suffix tensors are needed";
     if ((long long)a.B * (a.T / a.block + 1) * a.Ls >= (1LL << 32)) return "fused backward with suffixes: too many suffix rows";

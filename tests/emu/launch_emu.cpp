@@ -66,14 +66,23 @@ int fpk_static_scratch(void** ptr, const char** /*err*/) {
 // ones take on a real device (several sequences per workgroup, split sequences).
 int fpk_compute_units() { return 8; }
 
-int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& a, void* /*stream*/, const char** err) {
+int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const char** err) {
+  fpk::FusedBwdArgs a = args;
+  a.fold = a.block > 0 && a.Ls <= fpk::FB_SFX_ROWS;
   if (const char* why = fpk::check_fused_bwd(a)) {
     *err = why;
     return 1;
   }
+  if (a.fold) {
+    if (int rc = run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_fold_lds_bytes(),
+                          [&](char* l) { fpk::fused_bwd<fpk::FB_FOLD>(a, l, fprt::block_index()); }))
+      return rc;
+    const int pairs = a.B * (a.T / a.block + 1) * a.H;
+    return run_grid(fpk::SI_THREADS, pairs < 3 ? pairs : 3, fpk::si_lds_bytes(), [&](char* l) { fpk::suffix_intra_bwd(a, l); });
+  }
   return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(), [&](char* l) {
-    if (a.block > 0) fpk::fused_bwd<true>(a, l, fprt::block_index());
-    else fpk::fused_bwd<false>(a, l, fprt::block_index());
+    if (a.block > 0) fpk::fused_bwd<fpk::FB_STOPS>(a, l, fprt::block_index());
+    else fpk::fused_bwd<fpk::FB_PLAIN>(a, l, fprt::block_index());
   });
 }
 

@@ -131,6 +131,7 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     (1, 4, 128, 16, 1, 0.5),     # two chunks per block
     (1, 8, 64, 64, 1, None),     # block == chunk, suffixes as long as a chunk, no initial state
     (1, 3, 192, 1, 1, 0.3),      # three chunks per block, one-token suffixes
+    (2, 8, 64, 9, 2, 0.3),       # short suffixes folded into every chunk; 36 (suffix, head) pairs over 3 workgroups of the second kernel
 ])
 def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, block, Ls, H, state_std):
     """dk = dv = 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
