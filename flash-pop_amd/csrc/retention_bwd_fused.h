@@ -14,8 +14,10 @@
 //                         segment from the last to the first, close to the reverse workgroup of
 //                         its stream, so that rows read twice are read close together in time.
 //
-// With POP suffixes (the SFX instantiations) a suffix is one more stop of either walk at its block
-// boundary, with tensors of its own: it reads the state there and leaves it as it is.
+// With POP suffixes a suffix is one more stop of either walk at its block boundary, with tensors of
+// its own: it reads the state there and leaves it as it is (FB_STOPS).  Suffixes of at most 16 tokens
+// are not stops (FB_FOLD): the two things that tie a suffix to the carried states become part of the
+// chunk that starts at its boundary, and the rest is done by a second, small kernel (suffix_intra_bwd).
 //
 // Outputs are stored, and q (which only the reverse workgroup reads) is loaded, with the
 // non-temporal hint: kept out of the caches they leave room for k, v and dO, which both workgroups
@@ -454,9 +456,6 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   for (int it = 0; it < nitems; ++it) {
     const int L = cur.L;
     const bool sfx = SFX && cur.sfx;
-    // a suffix of at most 16 tokens lives in the first k-step of tokens and the first 32-token half:
-    // one score tile, one product each for the outputs and the state
-    const bool brief = sfx && L <= 16;
     const Item after = item_of(it + 2);
     // ---- the previous item's outputs leave (nothing writes the staging tiles before the next barrier)
     if (it > 0) {
@@ -479,7 +478,7 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       };
       constexpr int AHEAD = 3;   // k-steps of operands in flight
       if (sfx) {   // no read-out: only the score tile
-        if (scores && !(brief && rt != 0)) {
+        if (scores) {
 #pragma unroll
           for (int t = 0; t < 8; ++t) {
             wf[t] = frag_cols(s_wrow, t);
@@ -532,17 +531,6 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     // FOLD: the next chunk's suffix rows travel during this stretch only (registers are scarce in the first one)
     if constexpr (FOLD) pf_s = load_suffix(it + 1);
     // ---- stretch 2: Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]
-    if (brief) {
-      const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * rt), pq = ld128(xp_pass + lane * 8);
-      const u32x4 ua = frag_rows(Qs, tr_nat, 0, 32 * at_);
-      const u32x4 ub0 = frag_rows(Gs, tr_nat, 0, 32 * nt0), ub1 = frag_rows(Gs, tr_nat, 0, 32 * (nt0 + 1));
-      fprt::sched_fence();
-      acc[0] = fprt::mfma_32x32x16_bf16(za, pq, acc[0]);
-      const u32x4 wa = weigh(ua, wk0);
-      racc[0] = fprt::mfma_32x32x16_bf16(wa, ub0, racc[0]);
-      racc[1] = fprt::mfma_32x32x16_bf16(wa, ub1, racc[1]);
-      put_output(out, c, 32 * rt, g, acc[0]);
-    } else {
     {
       u32x4 za[4], pq0[4], pq1[2];
 #pragma unroll
@@ -593,7 +581,6 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
         }
         fprt::sched_fence();
       }
-    }
     }
     if constexpr (FOLD) {
       // the suffix at this chunk's first token: what it adds to dS is not decayed (it reads the state as it is there)
@@ -738,7 +725,6 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     const bool fresh = !SFX && next >= 0 && next != chunk_of(it) + 1;   // the next chunk starts another segment
     const bool sfx = SFX && cur.sfx;
     const int L = cur.L;
-    const bool brief = sfx && L <= 16;   // as in the reverse workgroup: first k-step of tokens, first half only
     const Item after = item_of(it + 2);
     if (it > 0) {   // nothing writes the staging tile before the next barrier
       drain_tile(k, OUT, p.dq, p.dq_sfx, prev);
@@ -746,7 +732,7 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     }
     f32x16 acc[2];
     if constexpr (state_role) {
-      if (rt < 3 && !(brief && rt != 0)) {
+      if (rt < 3) {
         ScoreFrags sf;
         f32x16 sc = {0};
 #pragma unroll
@@ -764,19 +750,7 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
       // Y^T[n][i] = gamma^(i+1) sum_a R^T[n][a] X[i][a]
       acc[0] = f32x16{0};
       acc[1] = f32x16{0};
-      if (brief) {
-        u32x4 ra[8], x0[8];
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          ra[t] = frag_cols(rrow, t);
-          x0[t] = frag_cols(xrow0, t);
-        }
-        fprt::sched_fence();
-#pragma unroll
-        for (int t = 0; t < 8; ++t) acc[0] = fprt::mfma_32x32x16_bf16(ra[t], x0[t], acc[0]);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[0][r] *= wread0;
-      } else {
+      {
       u32x4 ra[8], x0[8], x1[8];
       auto request = [&](int t) {
         ra[t] = frag_cols(rrow, t);
@@ -827,11 +801,7 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
     if constexpr (!state_role) {
       // Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]; tokens j < 32 reach both halves (tiles (0,0), (0,1)),
       // the others only the second
-      if (brief) {
-        const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * rt), pq = ld128(XP + lane * 8);
-        acc[0] = fprt::mfma_32x32x16_bf16(za, pq, acc[0]);
-        put_output(OUT, c, 32 * rt, g, acc[0]);
-      } else {
+      {
       u32x4 za[4], pq1[4], pq0[2];
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) {

@@ -15,7 +15,7 @@ import subprocess
 import sys
 from collections import defaultdict
 
-OURS = ("retention_", "segment_scan", "segment_contrib", "decode_step", "rotary_qk", "gated_norm")
+OURS = ("retention_", "suffix_intra", "segment_scan", "segment_contrib", "decode_step", "rotary_qk", "gated_norm")
 COPY_KIB = 1 << 20   # the calibration copies 1 GiB
 
 
@@ -53,7 +53,7 @@ def copy_reading(path, counter):
 
 
 FAMILIES = (
-    ("retention kernels of this library", ("retention_", "segment_scan", "segment_contrib", "decode_step")),
+    ("retention kernels of this library", ("retention_", "suffix_intra", "segment_scan", "segment_contrib", "decode_step")),
     ("rotary embedding kernel of this library", ("rotary_qk",)),
     ("norm + gate kernels of this library", ("gated_norm",)),
     ("GEMMs (rocBLAS / hipBLASLt)", ("Cijk_", "gemm", "Gemm")),
