@@ -175,9 +175,9 @@ int forward(const Shape& s, const void* q, const void* k, const void* v, const v
 
 // The plain backward with dk = dv = 128 has a kernel of its own that reads q, k, v, dO once for dk
 // and dv together (retention_bwd_fused.h); it runs two workgroups per (batch, head) stream, so it
-// is chosen when those fill at least half of the device.  FLASHPOP_BWD=passes / fused in the
-// environment overrides the choice (for A/B measurements).
-bool use_fused_backward(const Shape& s, const void* d_blocks) {
+// is chosen when there are enough streams for the device (below).  FLASHPOP_BWD=passes / fused in
+// the environment overrides the choice (for A/B measurements).
+bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes = false) {
   if (s.dk != fpk::FB_D || s.dv != fpk::FB_D || d_blocks) return false;
   if (s.T < 8 * fpk::CH) return false;   // short sequences: the walk over many of them per workgroup serves better
   if (const char* e = std::getenv("FLASHPOP_BWD")) {
@@ -185,8 +185,11 @@ bool use_fused_backward(const Shape& s, const void* d_blocks) {
     if (std::strcmp(e, "fused") == 0) return true;
   }
   // two workgroups per stream: with fewer than two thirds of the compute units covered the column-tiled
-  // passes, which fill the chip, are faster (256 units, T = 4096: 64 streams 0.33 ms against 0.30 ms; with POP
-  // suffixes, 80 streams 0.375 against 0.353 ms)
+  // passes, which fill the chip, are faster (256 units, T = 4096: 64 streams 0.33 ms against 0.30 ms).  With POP
+  // suffixes the passes pay for every suffix as a stop of each of their four walks and this kernel does not:
+  // it wins from 3/16 of the units' worth of streams on (48 streams, 64-token blocks: 0.44 against 0.57 ms; 512-token
+  // blocks: even between 48 and 80 streams; 32 streams: the passes by 8 %)
+  if (pop_suffixes) return 16LL * s.B * s.H >= 3LL * fpk_compute_units();
   return 3LL * s.B * s.H >= fpk_compute_units();
 }
 
@@ -458,7 +461,7 @@ int fused_backward(const Shape& s, const void* q, const void* k, const void* v, 
                    const double* decays, const void* d_o, const void* d_o_sfx, const void* d_s_out, void* dq, void* dk_,
                    void* dv_, void* dq_sfx, void* dk_sfx, void* dv_sfx, void* d_s0, int block, void* stream) {
   // whole 64-token chunks per block, suffixes of one chunk at most: the kernel that carries dS once
-  if (use_fused_backward(s, nullptr) && block % fpk::CH == 0 && s.T % block == 0 && x.len <= fpk::CH) {
+  if (use_fused_backward(s, nullptr, true) && block % fpk::CH == 0 && s.T % block == 0 && x.len <= fpk::CH) {
     const SuffixGrads sg{d_o_sfx, dq_sfx, dk_sfx, dv_sfx, block};
     return backward_fused(s, q, k, v, s0, decays, d_o, d_s_out, dq, dk_, dv_, d_s0, stream, nullptr, 0, &x, &sg);
   }
