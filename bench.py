@@ -197,7 +197,7 @@ def gpu_leg(args):
         torch.cuda.synchronize()
         pop_ms = (time.perf_counter() - t0) * 1e3 / n
 
-        # the same work in one walk per pass: suffixes read the state at their boundary in place
+        # the same work with the suffixes inside the walks: they read the state at their boundary in place
         def fused_step():
             o, o_s, _ = flash_pop_retention_with_suffixes(*leaves, s, decays, block, *sleaves)
             return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
@@ -217,7 +217,7 @@ def gpu_leg(args):
             "tokens": tok_ctx + tok_sfx,
             "ms_per_step": round(fused_ms, 4),
             "cost_per_token_vs_plain": ratio(fused_ms),
-            "path": "flash_pop_retention_with_suffixes (one walk per pass)",
+            "path": "flash_pop_retention_with_suffixes (suffixes read the state at their boundary in place: no block state in HBM)",
             "two_op_path": {
                 "path": "flash_pop_retention, torch.cat of the block states, fused_chunk_retention (the reference's call sequence)",
                 "ms_per_step": round(pop_ms, 4),
