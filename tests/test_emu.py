@@ -110,7 +110,7 @@ def test_fused_pop_fwd_bwd(emu_lib, B, nblk, block, Ls, H, dk, dv, state_std, ta
     (1, 512, 1, 256, 64, 0.5, 2),      # 256-wide keys: the state-only walk visits every chunk twice
     (1, 512, 1, 192, 64, 0.5, 2),      # 192-wide keys: three visits
     (1, 640, 1, 128, 128, 0.5, 2),     # 128-wide keys: the state-only kernel with the whole state tile per workgroup, 5 chunks
-    (1, 1024, 1, 128, 256, None, 4),   # ... two workgroups per sequence (256-wide values), 4 chunks per segment
+    (1, 512, 1, 128, 256, None, 2),    # ... two workgroups per sequence (256-wide values), 4 chunks per segment
 ])
 def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     decays = (0.97,) * H
@@ -130,8 +130,8 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
 @pytest.mark.parametrize("B,nblk,block,Ls,H,state_std", [
     (1, 4, 128, 16, 1, 0.5),     # two chunks per block
     (1, 8, 64, 64, 1, None),     # block == chunk, suffixes as long as a chunk, no initial state
-    (1, 3, 192, 1, 1, 0.3),      # three chunks per block, one-token suffixes
-    (2, 8, 64, 9, 2, 0.3),       # short suffixes folded into every chunk; 36 (suffix, head) pairs over 3 workgroups of the second kernel
+    (1, 3, 192, 1, 2, 0.3),      # three chunks per block, one-token suffixes, two heads
+    (1, 8, 64, 9, 1, 0.3),       # short suffixes folded into every chunk; 9 suffixes over 3 workgroups of the second kernel
 ])
 def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, block, Ls, H, state_std):
     """dk = dv = 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
