@@ -67,6 +67,8 @@ def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, ora
     (1, 3, 64, 16, 2, 256, 128),     # 256-wide keys: two visits per chunk in the forward and dv passes
     (1, 2, 96, 24, 2, 128, 256),     # 256-wide values: two visits per chunk in the dq and dk passes
     (2, 3, 64, 16, 2, 192, 192),     # 192-wide keys and values: three visits per chunk in every pass
+    (3, 8, 64, 16, 16, 128, 128),    # 48 streams: the fewest that take the backward with the suffixes folded into the chunks
+    (3, 4, 128, 33, 16, 128, 128),   # ... with suffixes too long to fold: stops of its walks
 ])
 def test_fused_parity_sweep(B, N, block, Ls, H, dk, dv):
     run_fused(B, N, block, Ls, H, dk, dv, 0.3, seed=N * block + Ls, decay_range=(5, 12))
@@ -90,6 +92,22 @@ def test_fused_trailing_tokens_and_long_suffixes(B, N, block, Ls, H, dk, dv, tai
     # build its suffix call from, pop_retnet.py:161-164, and the oracle follows it: zeros instead)
     run_fused(B, N, block, Ls, H, dk, dv, None if N else 0.0, seed=N * block + Ls + tail + 1, decay_range=(5, 12), tail=tail,
               d_last=False)
+
+
+def test_folded_suffix_backward_is_deterministic():
+    """Two runs of the fused POP backward (dk = dv = 128, 16-token suffixes: two launches, no atomics) give the same bits."""
+    from flash_pop_amd import _lib
+    lib = _lib.load()
+    B, N, block, Ls, H = 4, 16, 64, 16, 16
+    decays = oracle.head_decays(H)
+    q, k, v, s = hp.make_inputs(B, N * block, H, 128, 128, seed=71, state_std=0.2, device=DEV)
+    sfx = hp.make_suffix_inputs(B, N, Ls, H, 128, 128, seed=72, device=DEV)
+    cot = hp.make_cotangents([(B, N * block, H, 128), tuple(sfx[2].shape), (B, H, 128, 128)], seed=73, device=DEV)
+    first = hp.raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot)
+    second = hp.raw_fused_bwd(lib, q, k, v, s, sfx, decays, block, cot)
+    torch.cuda.synchronize()
+    for name, x, y in zip(("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0"), first, second):
+        assert torch.equal(x, y), name
 
 
 def test_fused_without_state_and_without_last_state_gradient():
