@@ -4,10 +4,14 @@ A step is one forward + backward of fused_chunk_retention over one synthetic bat
 benchmark configuration 2 (bf16, B=8 H=16 T=4096 dk=dv=128, zero initial state, dO ~ N(0,1)), inputs
 resident in HBM.  Prints ONE JSON line: whole-job TFLOP/s from the algorithmic FLOP count
 (dense chunk-64 tiles, no recompute), tokens/s, the HBM roofline of the backward kernel (the
-dominant launch of a step) measured with events on the launch stream, and the CPU oracle timed on
-the host cores beside it.
+dominant launch of a step) measured with events on the launch stream, the same step timed from
+an idle device, the other benchmark configurations each with a roofline object of its own, and
+the CPU oracle timed on the host cores beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--spin-up S] [--no-cpu] [--no-pop] [--no-long] [--no-layer] [--no-model]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--spin-up S] [--no-cpu] [--no-pop] [--no-long]
+                    [--no-layer5] [--no-layer] [--no-model]
+    python bench.py --profile-leg {headline,pop_fused,pop_two_op,long,layer5} --steps K
+        exactly K steps of one workload and nothing else: what the rocprofv3 runs of profile_counters.sh trace
 """
 import argparse
 import json
@@ -16,9 +20,10 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for p in (ROOT, os.path.join(ROOT, "flash-pop_amd"), os.path.join(ROOT, "tests")):
+for p in (ROOT, os.path.join(ROOT, "flash-pop_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
+TESTS = os.path.join(ROOT, "tests")     # the model harness and (CPU leg only) the oracle's helpers live there
 
 CHUNK = 64
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
@@ -30,13 +35,23 @@ def profiled_traffic(kernel):
     """HBM bytes per launch of `kernel` at config 2 as the hardware counters gave them (FETCH_SIZE and
     WRITE_SIZE, each scaled by what it reads for a plain copy of known size).  The figure is not
     measured by this script: it is read from the summary under profiles/ that the counter runs
-    of flash-pop_amd/profile_counters.sh produced, together with the commit it was measured at.
+    of profile_counters.sh produced, together with the commit it was measured at.
     -> (bytes or None, commit or None)"""
+    return _profile_line(r"^HBM_TRAFFIC %s bytes_per_launch=(\d+) measured_at=(\w+)", kernel)
+
+
+def profiled_step_traffic(leg):
+    """HBM bytes per step of a whole workload (all its launches), from the same counter runs:
+    `HBM_TRAFFIC_STEP <leg> bytes_per_step=<n> measured_at=<commit>`.  -> (bytes or None, commit or None)"""
+    return _profile_line(r"^HBM_TRAFFIC_STEP %s bytes_per_step=(\d+) measured_at=(\w+)", leg)
+
+
+def _profile_line(pattern, name):
     import glob
     import re
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
         with open(path) as f:
-            m = re.search(r"^HBM_TRAFFIC %s bytes_per_launch=(\d+) measured_at=(\w+)" % re.escape(kernel), f.read(), re.M)
+            m = re.search(pattern % re.escape(name), f.read(), re.M)
         if m:
             return int(m.group(1)), m.group(2)
     return None, None
@@ -69,20 +84,46 @@ def algorithmic_bytes(B, T, H, dk, dv):
     return 2 * (2 * dk + 2 * dv) * n, 2 * (4 * dk + 3 * dv) * n
 
 
-def gpu_leg(args):
-    import torch
-    import oracle
-    import helpers as hp
-    from flash_pop_amd import fused_chunk_retention, flash_pop_retention, _lib
-    from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
+def head_decays(H):
+    """gamma_h = 1 - 2^(-5-h) (flash_pop/retnet.py:70-76), as Python floats."""
+    return tuple(1.0 - 2.0 ** (-5.0 - h) for h in range(H))
 
-    _lib.load()   # fail loudly before any timing if the HIP library is missing
-    dev = "cuda:0"
+
+def make_inputs(B, T, H, dk, dv, seed, state_std=None, device="cpu"):
+    """q, k, v ~ N(0,1) in bf16 (k is scaled by dk^-1/2 inside the op), generated on the host so that the
+    CPU baseline sees the same bits; state_std None: no state, 0: zeros, else N(0, std^2)."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, T, H, dk, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, T, H, dk, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, T, H, dv, generator=g).to(torch.bfloat16)
+    if state_std is None:
+        s = None
+    elif state_std == 0:
+        s = torch.zeros(B, H, dk, dv, dtype=torch.bfloat16)
+    else:
+        s = (torch.randn(B, H, dk, dv, generator=g) * state_std).to(torch.bfloat16)
+    return tuple(None if t is None else t.to(device) for t in (q, k, v, s))
+
+
+def make_cotangents(shapes, seed, device="cpu"):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(*s, generator=g).to(torch.bfloat16).to(device) for s in shapes]
+
+
+# ---- the workloads: each returns step(ev=None) -> None and a description; ev = three events recorded before the
+# forward, between forward and backward and after the backward, on the stream the kernels are launched on -----------
+
+def workload_headline(dev):
+    """Config 2: plain retention forward + backward, zero initial state (the caller's zeros: no gradient)."""
+    import torch
+    from flash_pop_amd import fused_chunk_retention
     B, T, H, dk, dv = 8, 4096, 16, 128, 128
-    decays = oracle.head_decays(H)
-    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0, device=dev)
-    d_o, = hp.make_cotangents([(B, T, H, dv)], seed=1, device=dev)
-    leaves = [t.requires_grad_() for t in (q, k, v)]   # the state is the caller's zeros: no gradient
+    decays = head_decays(H)
+    q, k, v, s = make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0, device=dev)
+    d_o, = make_cotangents([(B, T, H, dv)], seed=1, device=dev)
+    leaves = [t.requires_grad_() for t in (q, k, v)]
 
     def step(ev=None):
         if ev:
@@ -90,29 +131,152 @@ def gpu_leg(args):
         o, S = fused_chunk_retention(*leaves, s, decays)
         if ev:
             ev[1].record()
-        grads = torch.autograd.grad([o], leaves, [d_o])
+        torch.autograd.grad([o], leaves, [d_o])
         if ev:
             ev[2].record()
-        return grads
 
+    b = algorithmic_bytes(B, T, H, dk, dv)
+    return step, {"shape": (B, T, H, dk, dv), "tokens": B * T, "bytes": b, "flops": algorithmic_flops(B, T, H, dk, dv)}
+
+
+def _pop_workload(dev, B, T, H, dk, dv, block, Ls, fused, seeds):
+    import torch
+    from flash_pop_amd import fused_chunk_retention, flash_pop_retention
+    from flash_pop_amd.pop_retention import flash_pop_retention_with_suffixes
+    decays = head_decays(H)
+    N = T // block
+    q, k, v, s = make_inputs(B, T, H, dk, dv, seed=seeds[0], state_std=0.0, device=dev)
+    d_o, = make_cotangents([(B, T, H, dv)], seed=seeds[1], device=dev)
+    qs, ks, vs, _ = make_inputs(B * (N + 1), Ls, H, dk, dv, seed=seeds[2], device=dev)
+    d_os, = make_cotangents([(B * (N + 1), Ls, H, dv)], seed=seeds[3], device=dev)
+    leaves = [t.requires_grad_() for t in (q, k, v)]
+    sleaves = [t.requires_grad_() for t in (qs, ks, vs)]
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        if fused:   # the suffixes inside the walks: they read the state at their boundary in place
+            o, o_s, _ = flash_pop_retention_with_suffixes(*leaves, s, decays, block, *sleaves)
+        else:       # the reference's call sequence
+            o, states = flash_pop_retention(*leaves, s, decays, block)
+            starts = torch.cat((s[:, None], states), dim=1).flatten(0, 1)
+            o_s, _ = fused_chunk_retention(*sleaves, starts, decays)
+        if ev:
+            ev[1].record()
+        torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
+        if ev:
+            ev[2].record()
+
+    tok_ctx, tok_sfx = B * T, B * (N + 1) * Ls
+    # every token of the context and of the suffixes once per tensor; the states stay on chip in the fused op
+    b = algorithmic_bytes(1, tok_ctx + tok_sfx, H, dk, dv)
+    return step, {"shape": (B, T, H, dk, dv), "tokens": tok_ctx + tok_sfx, "tokens_context": tok_ctx, "bytes": b}
+
+
+def workload_pop_fused(dev):
+    """Config 4 through flash_pop_retention_with_suffixes: 64-token blocks, 65 suffixes of 16 tokens per sequence."""
+    return _pop_workload(dev, 8, 4096, 16, 128, 128, 64, 16, True, (0, 1, 2, 3))
+
+
+def workload_pop_two_op(dev):
+    """Config 4 through flash_pop_retention, torch.cat of the block states and fused_chunk_retention on the suffix batch."""
+    return _pop_workload(dev, 8, 4096, 16, 128, 128, 64, 16, False, (0, 1, 2, 3))
+
+
+def workload_layer5(dev):
+    """The retention op of one layer of config 5's model: B=8 T=2048 H=12 dk=64 dv=128, 64-token blocks,
+    33 suffixes of 16 tokens per sequence, through flash_pop_retention_with_suffixes."""
+    return _pop_workload(dev, 8, 2048, 12, 64, 128, 64, 16, True, (10, 11, 12, 13))
+
+
+def workload_long(dev):
+    """Config 3: B=2 H=8 T=16384 dk=128 dv=256 with a carried state and its gradient.  16 streams cannot fill 256
+    compute units, so the op cuts each sequence into segments (fp_retention_*_split)."""
+    import torch
+    from flash_pop_amd import fused_chunk_retention
+    B, T, H, dk, dv = 2, 16384, 8, 128, 256
+    decays = head_decays(H)
+    q, k, v, s = make_inputs(B, T, H, dk, dv, seed=4, state_std=0.02, device=dev)
+    d_o, d_s = make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=5, device=dev)
+    leaves = [t.requires_grad_() for t in (q, k, v, s)]
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        o, S = fused_chunk_retention(*leaves, decays)
+        if ev:
+            ev[1].record()
+        torch.autograd.grad([o, S], leaves, [d_o, d_s])
+        if ev:
+            ev[2].record()
+
+    return step, {"shape": (B, T, H, dk, dv), "tokens": B * T, "bytes": algorithmic_bytes(B, T, H, dk, dv),
+                  "flops": algorithmic_flops(B, T, H, dk, dv)}
+
+
+WORKLOADS = {"headline": workload_headline, "pop_fused": workload_pop_fused, "pop_two_op": workload_pop_two_op,
+             "long": workload_long, "layer5": workload_layer5}
+
+
+def time_steps(step, n):
+    """n steps bracketed by synchronisations -> (wall ms per step, forward ms, backward ms from the events)."""
+    import torch
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(n)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(n):
+        step(events[i])
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / n
+    return wall, sum(e[0].elapsed_time(e[1]) for e in events) / n, sum(e[1].elapsed_time(e[2]) for e in events) / n
+
+
+def settle_and_time(step, args, n, warm):
+    if args.spin_up > 0:   # (inputs are made on the host: the device idled meanwhile and its clocks fell back)
+        spin_up(step, args.spin_up)
+    for _ in range(warm):
+        step()
+    return time_steps(step, n)
+
+
+def step_roofline(leg, info, ms, fwd_ms, bwd_ms, kernels):
+    """The HBM roofline of a whole step of a workload: its algorithmic bytes (every tensor once per pass) over
+    its time, the forward and backward parts from events on the launch stream, and the HBM traffic of all
+    its launches as the counters gave it (read from profiles/)."""
+    b_fwd, b_bwd = info["bytes"]
+    traffic, commit = profiled_step_traffic(leg)
+    gbs = lambda nbytes, t: round(nbytes / (t * 1e-3) / 1e9, 1)
+    return {
+        "bound": "hbm", "achieved": gbs(b_fwd + b_bwd, ms), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round((b_fwd + b_bwd) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "traffic": traffic, "traffic_measured_at_commit": commit,
+        "algorithmic_bytes_per_step": b_fwd + b_bwd, "kernels": kernels,
+        "forward_ms": round(fwd_ms, 4), "forward_achieved": gbs(b_fwd, fwd_ms),
+        "backward_ms": round(bwd_ms, 4), "backward_achieved": gbs(b_bwd, bwd_ms),
+    }
+
+
+def gpu_leg(args):
+    import torch
+    from flash_pop_amd import _lib
+
+    lib = _lib.load()   # fail loudly before any timing if the HIP library is missing
+    dev = "cuda:0"
+    step, info = workload_headline(dev)
+    B, T, H, dk, dv = info["shape"]
+
+    # the flags as given, from an idle device (the inputs were just made on the host): W warm-up steps, K timed
+    for _ in range(args.warmup):
+        step()
+    cold_ms, cold_fwd, cold_bwd = time_steps(step, args.steps)
+    # ... and with the device's clocks settled
     spin_steps = spin_up(step, args.spin_up) if args.spin_up > 0 else 0
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(events[i])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    # events on the stream the kernels are launched on (torch's current stream): the forward
-    # launch lies between the first two of a step, the backward launch between the last two
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
-    ms_per_step = wall * 1e3 / args.steps
+    ms_per_step, fwd_ms, bwd_ms = time_steps(step, args.steps)
 
-    f_fwd, f_bwd = algorithmic_flops(B, T, H, dk, dv)
-    b_fwd, b_bwd = algorithmic_bytes(B, T, H, dk, dv)
+    f_fwd, f_bwd = info["flops"]
+    b_fwd, b_bwd = info["bytes"]
     tflops = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
     # A step is two launches: the forward pass and the whole backward in one kernel, which is the
     # dominant one (about 70 % of the step).  Its roofline: the bytes the backward has to move
@@ -143,9 +307,15 @@ def gpu_leg(args):
         "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         # the same time priced with only the causal half of every C x C tile counted (C -> (C + 1) / 2)
         "tflops_causal_only": round(sum(algorithmic_flops(B, T, H, dk, dv, C=(CHUNK + 1) / 2)) / (ms_per_step * 1e-3) / 1e12, 2),
+        # the same W + K steps started from an idle device, before the spin-up: what a cold call costs
+        "ms_per_step_cold": round(cold_ms, 4),
+        "value_cold": round((f_fwd + f_bwd) / (cold_ms * 1e-3) / 1e12, 2),
+        "fwd_ms_cold": round(cold_fwd, 4),
+        "bwd_ms_cold": round(cold_bwd, 4),
         "set_up": {"spin_up_seconds": args.spin_up, "spin_up_steps": spin_steps,
-                   "why": "device clocks settle over the first ~50 steps from idle; set-up ends with this much of the "
-                          "same work, then the --warmup steps, then the timed --steps"},
+                   "why": "device clocks settle over the first ~50 steps from idle; `value` is timed after this much of "
+                          "the same work and the --warmup steps, `value_cold` / `ms_per_step_cold` before it"},
+        "library_version": lib.fp_version(),
         "roofline": {
             "bound": "hbm",
             "kernel": bwd_kernel + " (one launch = the whole backward of a step: dq, dk, dv)",
@@ -155,6 +325,8 @@ def gpu_leg(args):
             "frac": round(bwd_gbs / HBM_PEAK_GBS, 4),
             "traffic": traffic,
             "traffic_measured_at_commit": traffic_commit,
+            # the counters' bytes over this run's launch time: the rate at which the kernel really streams
+            "achieved_on_measured_traffic": round(traffic / (bwd_ms * 1e-3) / 1e9, 1) if traffic else None,
             "launch_ms": round(bwd_ms, 4),
             "algorithmic_bytes_per_launch": b_bwd,
             # the other launch of a step and the step as a whole, priced the same way
@@ -168,98 +340,60 @@ def gpu_leg(args):
             "step_frac": round(step_gbs / HBM_PEAK_GBS, 4),
         },
     }
+    del step
+    n_other, warm_other = max(12, args.steps // 4), max(5, args.warmup // 2)
 
     if not args.no_pop:
-        # POP (config 4): context through flash_pop_retention with 64-token blocks, 65 suffixes of
-        # 16 tokens per sequence through fused_chunk_retention from the block states.
-        block, Ls = 64, 16
-        N = T // block
-        qs, ks, vs, _ = hp.make_inputs(B * (N + 1), Ls, H, dk, dv, seed=2, device=dev)
-        d_os, = hp.make_cotangents([(B * (N + 1), Ls, H, dv)], seed=3, device=dev)
-        sleaves = [t.requires_grad_() for t in (qs, ks, vs)]
-
-        def pop_step():
-            o, states = flash_pop_retention(*leaves, s, decays, block)
-            starts = torch.cat((s[:, None], states), dim=1).flatten(0, 1)
-            o_s, _ = fused_chunk_retention(*sleaves, starts, decays)
-            return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
-
-        # (the inputs of this leg were made on the host: the device idled meanwhile and its clocks fell back)
-        if args.spin_up > 0:
-            spin_up(pop_step, args.spin_up)
-        for _ in range(max(5, args.warmup // 2)):
-            pop_step()
-        torch.cuda.synchronize()
-        n = max(12, args.steps // 4)
-        t0 = time.perf_counter()
-        for _ in range(n):
-            pop_step()
-        torch.cuda.synchronize()
-        pop_ms = (time.perf_counter() - t0) * 1e3 / n
-
-        # the same work with the suffixes inside the walks: they read the state at their boundary in place
-        def fused_step():
-            o, o_s, _ = flash_pop_retention_with_suffixes(*leaves, s, decays, block, *sleaves)
-            return torch.autograd.grad([o, o_s], leaves + sleaves, [d_o, d_os])
-
-        for _ in range(max(5, args.warmup // 2)):
-            fused_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(n):
-            fused_step()
-        torch.cuda.synchronize()
-        fused_ms = (time.perf_counter() - t0) * 1e3 / n
-        tok_ctx, tok_sfx = B * T, B * (N + 1) * Ls
-        ratio = lambda ms: round((ms / (tok_ctx + tok_sfx)) / (ms_per_step / tok_ctx), 3)
+        ratio = lambda ms, i: round((ms / i["tokens"]) / (ms_per_step / i["tokens_context"]), 3)
+        step, i = workload_pop_two_op(dev)
+        two_ms, two_fwd, two_bwd = settle_and_time(step, args, n_other, warm_other)
+        two = {
+            "path": "flash_pop_retention, torch.cat of the block states, fused_chunk_retention (the reference's call sequence)",
+            "ms_per_step": round(two_ms, 4),
+            "cost_per_token_vs_plain": ratio(two_ms, i),
+            "roofline": step_roofline("pop_two_op", i, two_ms, two_fwd, two_bwd,
+                                      "context forward / backward with block states, suffix-batch forward / backward, torch's cat and slice copies"),
+        }
+        del step
+        step, i = workload_pop_fused(dev)
+        fused_ms, fused_fwd, fused_bwd = settle_and_time(step, args, n_other, warm_other)
         out["pop"] = {
             "workload": "config 4: POP context (64-token blocks) + 65 suffixes x 16 tokens per sequence, fwd+bwd",
-            "tokens": tok_ctx + tok_sfx,
+            "tokens": i["tokens"],
             "ms_per_step": round(fused_ms, 4),
-            "cost_per_token_vs_plain": ratio(fused_ms),
+            "cost_per_token_vs_plain": ratio(fused_ms, i),
             "path": "flash_pop_retention_with_suffixes (suffixes read the state at their boundary in place: no block state in HBM)",
-            "two_op_path": {
-                "path": "flash_pop_retention, torch.cat of the block states, fused_chunk_retention (the reference's call sequence)",
-                "ms_per_step": round(pop_ms, 4),
-                "cost_per_token_vs_plain": ratio(pop_ms),
-            },
+            "roofline": step_roofline("pop_fused", i, fused_ms, fused_fwd, fused_bwd,
+                                      "suffix walk of the pass kernel (forward); fused backward with folded suffixes + suffix_intra_bwd_kernel"),
+            "two_op_path": two,
         }
+        del step
     if not args.no_long:
-        # Long context, few streams (config 3): B=2 H=8 T=16384 dk=128 dv=256 with a carried state and
-        # its gradient.  16 streams cannot fill 256 compute units, so the op cuts each sequence into
-        # segments (fp_retention_*_split).
-        del leaves, q, k, v
-        B3, T3, H3, dk3, dv3 = 2, 16384, 8, 128, 256
-        dec3 = oracle.head_decays(H3)
-        q3, k3, v3, s3 = hp.make_inputs(B3, T3, H3, dk3, dv3, seed=4, state_std=0.02, device=dev)
-        d_o3, d_s3 = hp.make_cotangents([(B3, T3, H3, dv3), (B3, H3, dk3, dv3)], seed=5, device=dev)
-        l3 = [t.requires_grad_() for t in (q3, k3, v3, s3)]
-
-        def long_step():
-            o, S = fused_chunk_retention(*l3, dec3)
-            return torch.autograd.grad([o, S], l3, [d_o3, d_s3])
-
-        if args.spin_up > 0:
-            spin_up(long_step, args.spin_up)
-        for _ in range(max(5, args.warmup // 2)):
-            long_step()
-        torch.cuda.synchronize()
-        n = max(12, args.steps // 4)
-        t0 = time.perf_counter()
-        for _ in range(n):
-            long_step()
-        torch.cuda.synchronize()
-        long_ms = (time.perf_counter() - t0) * 1e3 / n
-        f3 = sum(algorithmic_flops(B3, T3, H3, dk3, dv3))
-        b3 = sum(algorithmic_bytes(B3, T3, H3, dk3, dv3))
+        step, i = workload_long(dev)
+        long_ms, long_fwd, long_bwd = settle_and_time(step, args, n_other, warm_other)
+        B3, T3, H3, dk3, dv3 = i["shape"]
         out["long_context"] = {
             "workload": "config 3: B=2 H=8 T=16384 dk=128 dv=256, carried state, fwd+bwd incl. dS0",
             "ms_per_step": round(long_ms, 4),
-            "tflops": round(f3 / (long_ms * 1e-3) / 1e12, 2),
-            "algorithmic_gbs": round(b3 / (long_ms * 1e-3) / 1e9, 1),
-            "segments_per_sequence": _lib.load().fp_retention_workspace_bytes(B3, T3, H3, dk3, dv3)
-            // (4 * B3 * H3 * dk3 * dv3),
+            "tflops": round(sum(i["flops"]) / (long_ms * 1e-3) / 1e12, 2),
+            "algorithmic_gbs": round(sum(i["bytes"]) / (long_ms * 1e-3) / 1e9, 1),
+            "segments_per_sequence": lib.fp_retention_workspace_bytes(B3, T3, H3, dk3, dv3) // (4 * B3 * H3 * dk3 * dv3),
+            "roofline": step_roofline("long", i, long_ms, long_fwd, long_bwd,
+                                      "split-sequence entry points: state-only passes, segment scans, forward pass and the gradient kernels on the segments"),
         }
+        del step
+    if not args.no_layer5:
+        step, i = workload_layer5(dev)
+        l5_ms, l5_fwd, l5_bwd = settle_and_time(step, args, n_other, warm_other)
+        out["model_layer"] = {
+            "workload": "the retention op of one layer of config 5: fused POP step, B=8 T=2048 H=12 dk=64 dv=128, "
+                        "64-token blocks, 33 suffixes x 16 tokens per sequence, fwd+bwd",
+            "tokens": i["tokens"],
+            "ms_per_step": round(l5_ms, 4),
+            "roofline": step_roofline("layer5", i, l5_ms, l5_fwd, l5_bwd,
+                                      "suffix walk of the pass kernel (forward); the backward kernels of this shape"),
+        }
+        del step
     if not args.no_layer:
         out["layer_ops"] = layer_leg(args, dev)
     if not args.no_model:
@@ -273,6 +407,8 @@ def layer_leg(args, dev):
     stage as eager torch (the reference's call sequence)."""
     import torch
     import torch.nn.functional as F
+    if TESTS not in sys.path:
+        sys.path.insert(0, TESTS)
     import model_harness as mh
     from flash_pop_amd import XPos, gated_group_norm
 
@@ -320,6 +456,8 @@ def model_leg(args, dev):
     one POP training step (fwd+bwd, B=8, T=2048 in 64-token blocks with 16-token suffixes), then
     256 recurrent decode steps from the states it leaves."""
     import torch
+    if TESTS not in sys.path:
+        sys.path.insert(0, TESTS)
     import model_harness as mh
 
     cfg = mh.HarnessConfig()
@@ -394,6 +532,8 @@ def cpu_leg(sample_batch=8, reps=3):
     `sample_batch` of the 8 sequences of config 2.  Threads: what torch takes from the
     environment (OMP_NUM_THREADS, else every core the process may run on)."""
     import torch
+    if TESTS not in sys.path:
+        sys.path.insert(0, TESTS)
     import oracle
     import helpers as hp
 
@@ -401,9 +541,10 @@ def cpu_leg(sample_batch=8, reps=3):
     if "OMP_NUM_THREADS" not in os.environ:
         torch.set_num_threads(allowed)
     B, T, H, dk, dv = sample_batch, 4096, 16, 128, 128
-    decays = oracle.head_decays(H)
-    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0)
-    d_o, = hp.make_cotangents([(B, T, H, dv)], seed=1)
+    decays = head_decays(H)
+    assert decays == oracle.head_decays(H)
+    q, k, v, s = make_inputs(B, T, H, dk, dv, seed=0, state_std=0.0)
+    d_o, = make_cotangents([(B, T, H, dv)], seed=1)
     times = []
     for i in range(reps + 1):
         t0 = time.perf_counter()
@@ -436,7 +577,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-pop", action="store_true", help="skip the POP (config 4) timing")
     ap.add_argument("--no-long", action="store_true", help="skip the long-context (config 3) timing")
+    ap.add_argument("--no-layer5", action="store_true", help="skip the timing of config 5's retention op on its own")
     ap.add_argument("--no-layer", action="store_true", help="skip the timing of the rotary / norm + gate kernels")
+    ap.add_argument("--profile-leg", choices=sorted(WORKLOADS), default=None,
+                    help="run exactly --steps steps of one workload and nothing else (for the rocprofv3 runs)")
     ap.add_argument("--no-model", action="store_true", help="skip the model-level (config 5) timing")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy (scales the FETCH_SIZE / WRITE_SIZE counters)")
@@ -452,6 +596,16 @@ def main():
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+    if args.profile_leg:
+        import torch
+        step, _ = WORKLOADS[args.profile_leg]("cuda:0")
+        if args.spin_up > 0:   # for kernel traces at settled clocks; counter runs pass --spin-up 0
+            spin_up(step, args.spin_up)
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        print(json.dumps({"profile_leg": args.profile_leg, "steps": args.steps}))
+        return
     out = gpu_leg(args)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_leg()

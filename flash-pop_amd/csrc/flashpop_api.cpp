@@ -21,12 +21,14 @@
 // k, per-head normalisation with the swish gate) are kernels of their own.
 #include "../../include/flashpop_hip.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <cstdint>
 #include <cstdlib>
+#include <mutex>
 
 #include "pass_args.h"
 
@@ -45,11 +47,43 @@ int fail(int code, const char* fmt, ...) {
 
 bool dim_ok(int d) { return d == 64 || d == 128 || d == 192 || d == 256; }
 
+// Two measurement switches, read from the environment once per process (the first entry point that
+// looks) and changed afterwards only through fp_set_backward_choice:
+//   FLASHPOP_BWD   auto | passes | fused   which backward runs where both exist
+//   FLASHPOP_CKPT  tokens between the checkpoints that the forward leaves for the fused backward
+//                  (a multiple of 64; 0: none; unset: 512)
+// A value that is neither is an error of every entry point, not a silent default.
+enum BwdChoice { BWD_AUTO = 0, BWD_PASSES = 1, BWD_FUSED = 2 };
+constexpr int kDefaultCheckpointEvery = 8 * fpk::CH;
+std::atomic<int> g_bwd_choice{BWD_AUTO}, g_ckpt_every{kDefaultCheckpointEvery};
+std::once_flag g_env_once;
+char g_env_error[160] = "";
+
+void read_environment() {
+  std::call_once(g_env_once, [] {
+    if (const char* e = std::getenv("FLASHPOP_BWD")) {
+      if (std::strcmp(e, "passes") == 0) g_bwd_choice = BWD_PASSES;
+      else if (std::strcmp(e, "fused") == 0) g_bwd_choice = BWD_FUSED;
+      else if (std::strcmp(e, "auto") != 0 && *e)
+        std::snprintf(g_env_error, sizeof g_env_error, "FLASHPOP_BWD=%.40s: expected auto, passes or fused", e);
+    }
+    if (const char* e = std::getenv("FLASHPOP_CKPT")) {
+      char* end = nullptr;
+      const long n = std::strtol(e, &end, 10);
+      if (end == e || *end || n < 0 || n % fpk::CH != 0 || n > (1 << 24))
+        std::snprintf(g_env_error, sizeof g_env_error, "FLASHPOP_CKPT=%.40s: expected a non-negative multiple of %d", e, fpk::CH);
+      else g_ckpt_every = (int)n;
+    }
+  });
+}
+
 struct Shape {
   int B, T, H, dk, dv;
 };
 
 int check_shape(const Shape& s, const double* decays) {
+  read_environment();
+  if (g_env_error[0]) return fail(FP_ERR_BAD_CONFIG, "%s", g_env_error);
   if (!decays) return fail(FP_ERR_NULL_POINTER, "head_decays is NULL");
   if (s.B < 1 || s.T < 1 || s.H < 1) return fail(FP_ERR_BAD_SHAPE, "B, T, H must be >= 1 (got %d, %d, %d)", s.B, s.T, s.H);
   if (s.H > fpk::MAX_HEADS) return fail(FP_ERR_BAD_SHAPE, "H = %d exceeds the supported maximum %d", s.H, fpk::MAX_HEADS);
@@ -67,6 +101,14 @@ int check_shape(const Shape& s, const double* decays) {
     if (!(decays[h] > 0.0) || !(decays[h] <= 1.0))
       return fail(FP_ERR_BAD_DECAY, "head_decays[%d] = %g is outside (0, 1]", h, decays[h]);
   }
+  return FP_OK;
+}
+
+// The pass kernels must not be recorded into a HIP graph (instantiating a graph that holds them has
+// crashed the host process); the entry points that launch them refuse a capturing stream.
+int check_stream(void* stream, const char* what) {
+  if (fpk_stream_is_capturing(stream))
+    return fail(FP_ERR_LAUNCH, "%s: the stream is capturing a HIP graph; this entry point must be called eagerly", what);
   return FP_OK;
 }
 
@@ -175,15 +217,15 @@ int forward(const Shape& s, const void* q, const void* k, const void* v, const v
 
 // The plain backward with dk = dv = 128 has a kernel of its own that reads q, k, v, dO once for dk
 // and dv together (retention_bwd_fused.h); it runs two workgroups per (batch, head) stream, so it
-// is chosen when there are enough streams for the device (below).  FLASHPOP_BWD=passes / fused in
-// the environment overrides the choice (for A/B measurements).
+// is chosen when there are enough streams for the device (below).  The backward choice (FLASHPOP_BWD,
+// fp_set_backward_choice) overrides that (for A/B measurements).
 bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes = false) {
   if (s.dk != fpk::FB_D || s.dv != fpk::FB_D || d_blocks) return false;
   if (s.T < 8 * fpk::CH) return false;   // short sequences: the walk over many of them per workgroup serves better
-  if (const char* e = std::getenv("FLASHPOP_BWD")) {
-    if (std::strcmp(e, "passes") == 0) return false;
-    if (std::strcmp(e, "fused") == 0) return true;
-  }
+  read_environment();
+  const int choice = g_bwd_choice.load(std::memory_order_relaxed);
+  if (choice == BWD_PASSES) return false;
+  if (choice == BWD_FUSED) return true;
   // two workgroups per stream: with fewer than two thirds of the compute units covered the column-tiled
   // passes, which fill the chip, are faster (256 units, T = 4096: 64 streams 0.33 ms against 0.30 ms).  With POP
   // suffixes the passes pay for every suffix as a stop of each of their four walks and this kernel does not:
@@ -197,8 +239,8 @@ bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes 
 // Eight chunks: the checkpoints cost 1/16 of the forward's traffic, and the segment that the two
 // workgroups of a stream share stays within reach of the caches.
 int checkpoint_interval(const Shape& s) {
-  int every = 8 * fpk::CH;
-  if (const char* e = std::getenv("FLASHPOP_CKPT")) every = std::atoi(e) / fpk::CH * fpk::CH;
+  read_environment();
+  const int every = g_ckpt_every.load(std::memory_order_relaxed);
   if (every <= 0 || !use_fused_backward(s, nullptr) || s.T <= every) return 0;
   return every;
 }
@@ -503,6 +545,7 @@ int fp_retention_fwd(const void* q, const void* k, const void* v, const void* s0
                      void* s_out, int B, int T, int H, int dk, int dv, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_fwd")) return rc;
   if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
   return forward(s, q, k, v, s0, head_decays, o, s_out, nullptr, 0, stream);
 }
@@ -512,6 +555,7 @@ int fp_retention_bwd(const void* q, const void* k, const void* v, const void* s0
                      int H, int dk, int dv, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_bwd")) return rc;
   if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
     return fail(FP_ERR_NULL_POINTER, "q, k, v, d_o, dq, dk and dv must not be NULL");
   return backward(s, q, k, v, s0, head_decays, d_o, d_s_out, nullptr, 0, dq, dk_, dv_, d_s0, stream);
@@ -531,6 +575,7 @@ int fp_retention_fwd_ckpt(const void* q, const void* k, const void* v, const voi
                           void* s_out, void* checkpoints, int every, int B, int T, int H, int dk, int dv, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_fwd_ckpt")) return rc;
   if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
   if (!checkpoints || every <= 0) return forward(s, q, k, v, s0, head_decays, o, s_out, nullptr, 0, stream);
   if (every % fpk::CH != 0) return fail(FP_ERR_BAD_SHAPE, "the checkpoint interval must be a multiple of %d tokens (got %d)", fpk::CH, every);
@@ -542,6 +587,7 @@ int fp_retention_bwd_ckpt(const void* q, const void* k, const void* v, const voi
                           void* dv_, void* d_s0, int B, int T, int H, int dk, int dv, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_bwd_ckpt")) return rc;
   if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
     return fail(FP_ERR_NULL_POINTER, "q, k, v, d_o, dq, dk and dv must not be NULL");
   if (checkpoints && (every <= 0 || every % fpk::CH != 0))
@@ -563,6 +609,7 @@ int fp_retention_fwd_split(const void* q, const void* k, const void* v, const vo
                            size_t workspace_bytes_given, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_fwd_split")) return rc;
   if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
   const int segments = plan_forward(s);
   if (int rc = check_workspace(s, segments, workspace, workspace_bytes_given)) return rc;
@@ -575,6 +622,7 @@ int fp_retention_fwd_split_static(const void* q, const void* k, const void* v, c
                                   void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_fwd_split_static")) return rc;
   if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
   const int segments = plan_forward(s);
   if (segments <= 1) return forward(s, q, k, v, s0, head_decays, o, s_out, nullptr, 0, stream);
@@ -598,6 +646,7 @@ int fp_retention_bwd_split(const void* q, const void* k, const void* v, const vo
                            int forward_states_kept, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_retention_bwd_split")) return rc;
   if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
     return fail(FP_ERR_NULL_POINTER, "q, k, v, d_o, dq, dk and dv must not be NULL");
   const int segments = plan_backward(s);
@@ -612,6 +661,7 @@ int fp_pop_retention_fwd(const void* q, const void* k, const void* v, const void
                          void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_pop_retention_fwd")) return rc;
   if (block_size < 1) return fail(FP_ERR_BAD_SHAPE, "block_size must be >= 1 (got %d)", block_size);
   if (!q || !k || !v || !o) return fail(FP_ERR_NULL_POINTER, "q, k, v and o must not be NULL");
   if (!block_states && T / block_size > 0)
@@ -624,6 +674,7 @@ int fp_pop_retention_bwd(const void* q, const void* k, const void* v, const void
                          int B, int T, int H, int dk, int dv, int block_size, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_pop_retention_bwd")) return rc;
   if (block_size < 1) return fail(FP_ERR_BAD_SHAPE, "block_size must be >= 1 (got %d)", block_size);
   if (!q || !k || !v || !d_o || !dq || !dk_ || !dv_)
     return fail(FP_ERR_NULL_POINTER, "q, k, v, d_o, dq, dk and dv must not be NULL");
@@ -636,6 +687,7 @@ int fp_pop_fused_fwd(const void* q, const void* k, const void* v, const void* s0
                      int H, int dk, int dv, int block_size, int sfx_len, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_pop_fused_fwd")) return rc;
   if (int rc = check_fused(s, block_size, sfx_len)) return rc;
   if (!q || !k || !v || !o || !q_sfx || !k_sfx || !v_sfx || !o_sfx)
     return fail(FP_ERR_NULL_POINTER, "q, k, v, o and their suffix counterparts must not be NULL");
@@ -649,6 +701,7 @@ int fp_pop_fused_bwd(const void* q, const void* k, const void* v, const void* s0
                      void* d_s0, int B, int T, int H, int dk, int dv, int block_size, int sfx_len, void* stream) {
   const Shape s{B, T, H, dk, dv};
   if (int rc = check_shape(s, head_decays)) return rc;
+  if (int rc = check_stream(stream, "fp_pop_fused_bwd")) return rc;
   if (int rc = check_fused(s, block_size, sfx_len)) return rc;
   if (!q || !k || !v || !q_sfx || !k_sfx || !v_sfx || !d_o || !d_o_sfx || !dq || !dk_ || !dv_ || !dq_sfx || !dk_sfx ||
       !dv_sfx)
@@ -728,8 +781,18 @@ int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, voi
   return gated_norm(r, g, d_out, nullptr, d_r, d_g, rows, H, dv, eps, stream);
 }
 
+int fp_set_backward_choice(int choice, int checkpoint_every) {
+  read_environment();
+  if (choice < BWD_AUTO || choice > BWD_FUSED) return fail(FP_ERR_BAD_CONFIG, "backward choice %d: expected 0 (by shape), 1 (passes) or 2 (fused)", choice);
+  if (checkpoint_every >= 0 && checkpoint_every % fpk::CH != 0)
+    return fail(FP_ERR_BAD_CONFIG, "the checkpoint interval must be a multiple of %d tokens (got %d)", fpk::CH, checkpoint_every);
+  g_bwd_choice.store(choice, std::memory_order_relaxed);
+  if (checkpoint_every >= 0) g_ckpt_every.store(checkpoint_every, std::memory_order_relaxed);
+  return FP_OK;
+}
+
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1006; }
+int fp_version(void) { return 1007; }
 
 }  // extern "C"

@@ -157,6 +157,15 @@ int fpk_static_scratch(void** ptr, const char** err) {
   return 0;
 }
 
+int fpk_stream_is_capturing(void* stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
 // Compute units of the current device (cached per thread and device).
 int fpk_compute_units() {
   static thread_local int dev_cached = -1, cus = 0;

@@ -210,11 +210,14 @@ int fpk_launch_contrib(const fpk::ContribArgs& args, void* stream, const char** 
 
 // Bytes of the library's own scratch array (one per device, see fpk_static_scratch).
 namespace fpk {
-constexpr size_t STATIC_SCRATCH_BYTES = 8u << 20;
+constexpr size_t STATIC_SCRATCH_BYTES = 16u << 20;
 }
 // Address of the scratch array on the current device (device memory, 256-byte aligned,
 // fpk::STATIC_SCRATCH_BYTES long); looked up on the first call on each device, never allocated.
 int fpk_static_scratch(void** ptr, const char** err);
+
+// Nonzero if `stream` is recording a HIP graph (the CPU test harness: a flag that its tests set).
+int fpk_stream_is_capturing(void* stream);
 
 // Compute units of the current device (what the launcher sizes its grids against).
 int fpk_compute_units();

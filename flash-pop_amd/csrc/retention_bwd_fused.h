@@ -908,8 +908,8 @@ FP_DEVICE void fused_bwd(const FusedBwdArgs& p, char* lds, int block) {
 // D[i][j] = scale gamma^(i - j) for j <= i, A = D . (q_s k_s^T) and dA = D . (dO_s v_s^T), both rounded to bf16:
 //   dv_s = A^T dO_s,   dk_s = dA^T q_s,   dq_s += dA k_s   (dq_s holds the part that came from the carried state).
 // One workgroup of 4 waves takes the (suffix, head) pairs m = block, block + grid, ...: three score tiles by one wave
-// each, then every wave a 32-column slice of each of the three outputs; the next pair's rows are on their way in
-// registers meanwhile.  The three products are the dv pass, the dk pass and the dq pass of the chunk kernels above
+// each, then every wave a 32-column slice of each of the three outputs (the dq_s slice starts from what the first launch
+// wrote, so that the sum is rounded once); the next pair's rows are on their way in registers meanwhile.  The three products are the dv pass, the dk pass and the dq pass of the chunk kernels above
 // on one 16-token tile, and are written with their pieces.
 constexpr int SI_THREADS = 256;
 constexpr int si_lds_bytes() { return 2 * (7 * FB_SFX_TILE + 3 * FB_XP); }   // q, k, v, dO; dv, dk, dq; score tiles
@@ -959,7 +959,8 @@ FP_DEVICE void suffix_intra_bwd(const FusedBwdArgs& p, char* lds) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) st128(TL + x * FB_SFX_TILE + at(ld_row + 16 * u, 8 * ld_piece), cur.in[2 * x + u]);
     }
-    const u32x4 dq_state = cur.dq;
+    // what the carried state gave to dq_s waits in the dq staging tile: the product below is added to it in fp32
+    st128(OUT + 2 * FB_SFX_TILE + at(ld_row, 8 * ld_piece), cur.dq);
     load(m + fprt::grid_size(), cur);
     fprt::block_sync();
     if (wave < 3) {
@@ -984,18 +985,15 @@ FP_DEVICE void suffix_intra_bwd(const FusedBwdArgs& p, char* lds) {
       const uint16_t* const Zs = TL + (o == 0 ? 3 : o == 1 ? 0 : 1) * FB_SFX_TILE;
       const u32x4 za = frag_rows(Zs, tr_acc, 0, 32 * wave), pq = ld128(XP + o * FB_XP + lane * 8);
       f32x16 acc = {0};
+      if (o == 2) acc = get_state(OUT + 2 * FB_SFX_TILE, c, 32 * wave, g);   // same layout as put_output: [token][feature]
       acc = fprt::mfma_32x32x16_bf16(za, pq, acc);
       put_output(OUT + o * FB_SFX_TILE, c, 32 * wave, g, acc);
     }
     fprt::block_sync();
-    // rows < Ls leave; dq_s is the sum with what the carried state gave
+    // rows < Ls leave
     {
       const u32x4 dvv = ld128(OUT + at(ld_row, 8 * ld_piece)), dkv = ld128(OUT + FB_SFX_TILE + at(ld_row, 8 * ld_piece));
-      const u32x4 dqi = ld128(OUT + 2 * FB_SFX_TILE + at(ld_row, 8 * ld_piece));
-      u32x4 dqv;
-#pragma unroll
-      for (int d = 0; d < 4; ++d)
-        dqv[d] = fprt::pack_bf16x2(bf16_elem(dqi, 2 * d) + bf16_elem(dq_state, 2 * d), bf16_elem(dqi, 2 * d + 1) + bf16_elem(dq_state, 2 * d + 1));
+      const u32x4 dqv = ld128(OUT + 2 * FB_SFX_TILE + at(ld_row, 8 * ld_piece));
       const uint32_t off = (uint32_t)ld_row * rowp + ld_piece * 16;
       fprt::buf_store128_nt(view(p.dv_sfx, m, p.Ls), off, dvv);
       fprt::buf_store128_nt(view(p.dk_sfx, m, p.Ls), off, dkv);

@@ -32,6 +32,7 @@ SIGNATURES = {
     "fp_rotary_qk": [_P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
     "fp_gated_group_norm_fwd": [_P, _P, _P, _L, _I, _I, _F, _P],
     "fp_gated_group_norm_bwd": [_P, _P, _P, _P, _P, _L, _I, _I, _F, _P],
+    "fp_set_backward_choice": [_I, _I],
     "fp_last_error": [],
     "fp_version": [],
 }

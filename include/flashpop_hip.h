@@ -16,6 +16,10 @@
  *   - launches are asynchronous on `stream` (a hipStream_t, NULL = default stream)
  *   - returns 0 on success, a negative FP_ERR_* code otherwise; fp_last_error() then gives a
  *     message (thread-local).  No kernel is launched when an argument check fails.
+ *   - the retention, POP and split entry points must not be recorded into a HIP graph: they return
+ *     FP_ERR_LAUNCH when `stream` is capturing (instantiating a graph that holds their kernels has
+ *     crashed the host process).  The decode step, the rotary embedding and the norm + gate entry
+ *     points can be captured.
  *   - results are deterministic: no atomics, fixed reduction order
  */
 #ifndef FLASHPOP_HIP_H
@@ -33,6 +37,7 @@ extern "C" {
 #define FP_ERR_UNSUPPORTED_DIM (-3)
 #define FP_ERR_BAD_DECAY (-4)
 #define FP_ERR_LAUNCH (-5)
+#define FP_ERR_BAD_CONFIG (-6)
 
 /* Replaces the kernel call in FusedChunkRetention.forward
  * (flash_pop/fused_retention/__init__.py:13-31).
@@ -103,14 +108,13 @@ int fp_retention_bwd_split(const void* q, const void* k, const void* v, const vo
 
 /* fp_retention_fwd_split without a workspace argument and without any allocation.  It has no
  * counterpart in the reference; it is for callers that cannot allocate device memory at the call:
- * code under HIP graph capture set-up, tight serving loops, harnesses that forbid hipMalloc.  The
- * segment states live in an array inside the library's code object (8 MiB per device, held from
- * the first use of the library on that device until the process ends).  Same results as
- * fp_retention_fwd_split, bit for bit.  A shape whose segment states need more than 8 MiB
- * (fp_retention_workspace_bytes says how much; on a 256-CU device only dk = 256 can) is rejected
- * with FP_ERR_BAD_SHAPE.  Every call on
- * a device uses that device's one array: two calls that overlap in time on one device (different
- * streams or threads) race; calls on one stream are ordered and safe. */
+ * tight serving loops, harnesses that forbid hipMalloc.  The segment states live in an array inside
+ * the library's code object (16 MiB per device, held from the first use of the library on that
+ * device until the process ends).  Same results as fp_retention_fwd_split, bit for bit.  A shape
+ * whose segment states need more than 16 MiB (fp_retention_workspace_bytes says how much: 64 KiB x
+ * max(dk, dv) x compute units / 256, so 16 MiB at most on a device of 256 compute units) is rejected
+ * with FP_ERR_BAD_SHAPE.  Every call on a device uses that device's one array: two calls that overlap
+ * in time on one device (different streams or threads) race; calls on one stream are ordered and safe. */
 int fp_retention_fwd_split_static(const void* q, const void* k, const void* v, const void* s0,
                                   const double* head_decays, void* o, void* s_out, int B, int T, int H, int dk, int dv,
                                   void* stream);
@@ -192,6 +196,18 @@ int fp_gated_group_norm_fwd(const void* r, const void* g, void* out, long long r
                             void* stream);
 int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, void* d_r, void* d_g, long long rows, int H,
                             int dv, double eps, void* stream);
+
+/* Measurement switch; no counterpart in the reference.  Where a shape can run both the fused backward
+ * kernel and the pass-per-gradient backward, the library chooses by shape; this overrides it for the
+ * whole process until called again (A/B timing, tests of the path not chosen).
+ *   choice            0 by shape (default), 1 always the passes, 2 the fused kernel wherever it exists
+ *   checkpoint_every  tokens between the states fp_retention_checkpoint_bytes asks the forward to leave:
+ *                     a multiple of 64, 0 for none, negative to leave the current setting (default 512)
+ * The environment variables FLASHPOP_BWD (auto | passes | fused) and FLASHPOP_CKPT give the initial
+ * values; they are read once per process, and a value that is none of these makes every entry point
+ * return FP_ERR_BAD_CONFIG.  Not synchronised with calls in flight on other threads: a forward and its
+ * backward must run under the same setting. */
+int fp_set_backward_choice(int choice, int checkpoint_every);
 
 /* Message for the last nonzero return on this thread ("" if none). */
 const char* fp_last_error(void);

@@ -143,11 +143,11 @@ int main() {
   rc |= fused(1, 1, 80, 5, 1, 64, 128, 30);   // tokens after the last block boundary
   rc |= fused(1, 0, 90, 12, 1, 64, 64, 70);   // no full block
   rc |= fused(1, 2, 64, 100, 1, 128, 64);     // suffixes in two parts
-  setenv("FLASHPOP_BWD", "fused", 1);         // one stream would not take this path by itself
+  fp_set_backward_choice(2, -1);        // one stream would not take this path by itself
   rc |= fused(1, 8, 64, 16, 1, 128, 128);     // backward in the kernel that carries dS once, suffixes as extra stops
   rc |= plain(1, 530, 1, 128, 128, false);    // the same kernel without suffixes, ragged last chunk
   rc |= checkpointed(1, 600, 1, 128);         // ... with the forward's checkpoints
-  unsetenv("FLASHPOP_BWD");
+  fp_set_backward_choice(0, -1);
   rc |= decode(2, 3, 64, 128);
   rc |= decode(1, 1, 256, 256);
   rc |= rotary(3, 11, 2, 64, true);           // last workgroup partly idle

@@ -62,6 +62,11 @@ int fpk_static_scratch(void** ptr, const char** /*err*/) {
   return 0;
 }
 
+// A test can pretend that streams are capturing (the C entry points of the pass kernels must refuse then).
+static int g_emu_capturing = 0;
+extern "C" void emu_set_capturing(int on) { g_emu_capturing = on; }
+int fpk_stream_is_capturing(void* /*stream*/) { return g_emu_capturing; }
+
 // Pretends the chip has 8 compute units, so that small test shapes take the paths that large
 // ones take on a real device (several sequences per workgroup, split sequences).
 int fpk_compute_units() { return 8; }

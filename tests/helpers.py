@@ -125,8 +125,8 @@ LITERAL_CEILING = {"o": 0.06, "S": 0.005, "dq": 0.06, "dk": 0.06, "dv": 0.06, "d
 def check_literal(got, ref, name, record=None):
     """frac_outside under the literal rtol = atol = 2e-2, asserted against LITERAL_CEILING."""
     rep = error_report(got, ref)
-    kind = name.split("[")[0].split(" ")[-1].replace("_sfx", "")
-    ceiling = LITERAL_CEILING[kind]
+    kind = name.split("[")[0].split(" ")[-1]
+    ceiling = LITERAL_CEILING.get(kind, LITERAL_CEILING[kind.replace("_sfx", "")])
     print(f"[literal 2e-2] {name}: frac_outside={rep['frac_outside']:.3e} rms_ratio={rep['rms_ratio']:.3e} "
           f"rms_ref={rep['rms_ref']:.3g} (ceiling {ceiling})", flush=True)
     if record is not None:

@@ -31,7 +31,7 @@ def test_header_and_binding_agree(lib):
     assert names == sorted(_lib.SIGNATURES), (names, sorted(_lib.SIGNATURES))
     for n in names:
         assert hasattr(lib, n), f"{n} not exported"
-    assert lib.fp_version() == 1006
+    assert lib.fp_version() == 1007
 
 
 def test_argument_checks_return_codes(lib):
@@ -66,6 +66,34 @@ def test_argument_checks_return_codes(lib):
     assert lib.fp_pop_retention_bwd(p, p, p, null, dec, p, p, p, p, null, null, *ok_dims, 4, None) == -1
     big = (ctypes.c_double * 513)(*([0.9] * 513))
     assert lib.fp_retention_fwd(p, p, p, null, big, p, null, 1, 8, 513, 64, 64, None) == -2   # more than 512 heads
+
+
+def test_backward_choice_switch_checks_its_arguments(lib):
+    assert lib.fp_set_backward_choice(3, -1) == -6 and b"backward choice" in lib.fp_last_error()
+    assert lib.fp_set_backward_choice(0, 100) == -6 and b"multiple of 64" in lib.fp_last_error()
+    assert lib.fp_set_backward_choice(1, 256) == 0
+    n = ctypes.c_int(-1)
+    # the passes are forced: no checkpoints are asked for, whatever the shape
+    assert lib.fp_retention_checkpoint_bytes(8, 4096, 16, 128, 128, ctypes.byref(n)) == 0 and n.value == 0
+    assert lib.fp_set_backward_choice(2, 256) == 0
+    assert lib.fp_retention_checkpoint_bytes(1, 4096, 1, 128, 128, ctypes.byref(n)) == 2 * 16 * 128 * 128 and n.value == 256
+    assert lib.fp_set_backward_choice(0, 512) == 0
+
+
+def test_environment_switches_are_validated_once():
+    """FLASHPOP_BWD / FLASHPOP_CKPT are read once per process; a value that is neither of the
+    documented ones makes every entry point fail (checked in child processes: nothing is launched)."""
+    import subprocess
+    import sys
+    from flash_pop_amd import _lib
+    code = ("import ctypes, sys; sys.path.insert(0, %r); from flash_pop_amd import _lib; lib = _lib.load();"
+            "d = (ctypes.c_double * 1)(0.9); p = ctypes.c_void_p(0x1000);"
+            "rc = lib.fp_retention_fwd(None, p, p, None, d, p, None, 1, 8, 1, 64, 64, None);"
+            "print(rc, lib.fp_last_error().decode())") % os.path.dirname(os.path.dirname(_lib.LIB_PATH))
+    run = lambda env: subprocess.run([sys.executable, "-c", code], env={**os.environ, **env}, capture_output=True, text=True).stdout
+    assert run({"FLASHPOP_BWD": "fuse"}).startswith("-6 FLASHPOP_BWD=fuse")
+    assert run({"FLASHPOP_CKPT": "100"}).startswith("-6 FLASHPOP_CKPT=100")
+    assert run({"FLASHPOP_BWD": "passes", "FLASHPOP_CKPT": "256"}).startswith("-1 ")
 
 
 def test_python_wrappers_refuse_cpu_tensors():

@@ -21,6 +21,18 @@ def emu_lib():
     return _lib.bind(os.path.join(EMU_DIR, "libflashpop_emu.so"))
 
 
+@pytest.fixture
+def choose_backward(emu_lib):
+    """choose_backward(1 | 2): force the pass-per-gradient backward / the fused kernel for this test."""
+    def choose(choice, every=-1):
+        assert emu_lib.fp_set_backward_choice(choice, every) == 0
+    yield choose
+    assert emu_lib.fp_set_backward_choice(0, 512) == 0
+
+
+PASSES, FUSED = 1, 2
+
+
 def _check_all(pairs):
     for name, got, ref in pairs:
         if ref is not None:
@@ -133,7 +145,7 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     (1, 3, 192, 1, 2, 0.3),      # three chunks per block, one-token suffixes, two heads
     (1, 8, 64, 9, 1, 0.3),       # short suffixes folded into every chunk; 9 suffixes over 3 workgroups of the second kernel
 ])
-def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, block, Ls, H, state_std):
+def test_fused_pop_backward_that_carries_ds_once(emu_lib, choose_backward, B, nblk, block, Ls, H, state_std):
     """dk = dv = 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
     the kernel that walks backward once for dk and dv beside a forward walk for dq, with the
     suffixes as extra stops at the block boundaries.  Same results as the pass-per-gradient path."""
@@ -142,11 +154,11 @@ def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, 
     q, k, v, s = hp.make_inputs(B, T, H, 128, 128, seed=T + Ls, state_std=state_std)
     sfx = hp.make_suffix_inputs(B, nblk, Ls, H, 128, 128, seed=T + Ls + 1)
     cot = hp.make_cotangents([(B, T, H, 128), tuple(sfx[2].shape), (B, H, 128, 128)], seed=T + 2)
-    monkeypatch.setenv("FLASHPOP_BWD", "fused")
+    choose_backward(FUSED)
     grads = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
     _, _, _, g_ref = hp.oracle_fused(q, k, v, s, sfx, decays, block, cot)
     _check_all([(n, g, r) for n, g, r in zip(FUSED_NAMES, grads, g_ref)])
-    monkeypatch.setenv("FLASHPOP_BWD", "passes")
+    choose_backward(PASSES)
     other = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
     for name, x, y in zip(FUSED_NAMES, grads, other):
         if x is not None:
@@ -160,11 +172,11 @@ def test_fused_pop_backward_that_carries_ds_once(emu_lib, monkeypatch, B, nblk, 
     (1, 600, 1, 0.2, 1024),     # interval longer than the sequence: no checkpoint at all
     (1, 576, 1, 0.4, 0),        # no checkpoint buffer: the fused backward walks forward from s0
 ])
-def test_fused_backward_with_checkpoints(emu_lib, monkeypatch, B, T, H, state_std, every):
+def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, state_std, every):
     """dk = dv = 128 and at least eight chunks: the backward that carries dS once, beside the
     workgroup that re-runs the state from the checkpoints the forward left (segments taken from
     the last to the first)."""
-    monkeypatch.setenv("FLASHPOP_BWD", "fused")
+    choose_backward(FUSED)
     decays = oracle.head_decays(H)
     q, k, v, s = hp.make_inputs(B, T, H, 128, 128, seed=T, state_std=state_std)
     d_o, d_s = hp.make_cotangents([(B, T, H, 128), (B, H, 128, 128)], seed=T + 1)
@@ -183,18 +195,54 @@ def test_fused_backward_with_checkpoints(emu_lib, monkeypatch, B, T, H, state_st
     assert (ds0 is None and g2[3] is None) or torch.equal(ds0, g2[3])
 
 
-def test_checkpoint_size_query(emu_lib, monkeypatch):
+def test_c_entry_points_refuse_a_capturing_stream(emu_lib):
+    """The entry points that launch the pass kernels return FP_ERR_LAUNCH, before launching anything, when
+    their stream is recording a HIP graph (the harness's stand-in for hipStreamIsCapturing is a flag);
+    the decode step stays capturable."""
+    import ctypes
+    decays = oracle.head_decays(1)
+    q, k, v, s = hp.make_inputs(1, 70, 1, 64, 64, seed=1, state_std=0.5)
+    d_o, = hp.make_cotangents([(1, 70, 1, 64)], seed=2)
+    sfx = hp.make_suffix_inputs(1, 1, 8, 1, 64, 64, seed=3)
+    cot = hp.make_cotangents([(1, 70, 1, 64), tuple(sfx[2].shape), (1, 1, 64, 64)], seed=4)
+    calls = [
+        lambda: hp.raw_fwd(emu_lib, q, k, v, s, decays),
+        lambda: hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None),
+        lambda: hp.raw_pop_fwd(emu_lib, q, k, v, s, decays, 32),
+        lambda: hp.raw_pop_bwd(emu_lib, q, k, v, s, decays, 32, d_o, None),
+        lambda: hp.raw_fused_fwd(emu_lib, q, k, v, s, sfx, decays, 64),
+        lambda: hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, 64, cot),
+        lambda: hp.raw_split_fwd(emu_lib, q, k, v, s, decays),
+        lambda: hp.raw_split_bwd(emu_lib, q, k, v, s, decays, d_o, None),
+        lambda: hp.raw_ckpt_fwd_bwd(emu_lib, q, k, v, s, decays, d_o, None, 64),
+    ]
+    emu_lib.emu_set_capturing(1)
+    try:
+        for call in calls:
+            with pytest.raises(AssertionError, match="rc=-5: .*capturing a HIP graph"):
+                call()
+        o = torch.zeros(1, 70, 1, 64, dtype=hp.BF16)
+        rc = emu_lib.fp_retention_fwd_split_static(hp._p(q), hp._p(k), hp._p(v), hp._p(s), hp._dec(decays), hp._p(o), None,
+                                                  1, 70, 1, 64, 64, None)
+        assert rc == -5 and b"capturing" in emu_lib.fp_last_error()
+        hp.raw_decode_step(emu_lib, q[:, 0], k[:, 0], v[:, 0], s, decays)
+    finally:
+        emu_lib.emu_set_capturing(0)
+    hp.raw_fwd(emu_lib, q, k, v, s, decays)
+
+
+def test_checkpoint_size_query(emu_lib, choose_backward):
     """fp_retention_checkpoint_bytes: 0 where the fused backward would not run or the sequence is
     no longer than one interval, else B * (T / every) state matrices."""
     import ctypes
     every = ctypes.c_int(-1)
-    monkeypatch.setenv("FLASHPOP_BWD", "fused")
+    choose_backward(FUSED)
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 2 * 2 * (4096 // 512) * 4 * 128 * 128
     assert every.value == 512
     assert emu_lib.fp_retention_checkpoint_bytes(2, 512, 4, 128, 128, ctypes.byref(every)) == 0 and every.value == 0
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 64, 128, ctypes.byref(every)) == 0
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, None) > 0
-    monkeypatch.setenv("FLASHPOP_BWD", "passes")
+    choose_backward(PASSES)
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 0
 
 
