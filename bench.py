@@ -37,7 +37,7 @@ def profiled_traffic(kernel):
     measured by this script: it is read from the summary under profiles/ that the counter runs
     of profile_counters.sh produced, together with the commit it was measured at.
     -> (bytes or None, commit or None)"""
-    return _profile_line(r"^HBM_TRAFFIC %s bytes_per_launch=(\d+) measured_at=(\w+)", kernel)
+    return _profile_line(r"^HBM_TRAFFIC %s(?:<[^>]*>)? bytes_per_launch=(\d+) measured_at=(\w+)", kernel)
 
 
 def profiled_step_traffic(leg):
@@ -281,11 +281,11 @@ def gpu_leg(args):
     # A step is two launches: the forward pass and the whole backward in one kernel, which is the
     # dominant one (about 70 % of the step).  Its roofline: the bytes the backward has to move
     # (q, k, v, dO in; dq, dk, dv out, each once) over its launch duration.
-    bwd_kernel = "retention_bwd_fused_kernel"
+    bwd_kernel = "retention_bwd_fused_kernel<128, 128, 0>"
     bwd_gbs = b_bwd / (bwd_ms * 1e-3) / 1e9
     fwd_gbs = b_fwd / (fwd_ms * 1e-3) / 1e9
     step_gbs = (b_fwd + b_bwd) / (ms_per_step * 1e-3) / 1e9
-    traffic, traffic_commit = profiled_traffic(bwd_kernel)
+    traffic, traffic_commit = profiled_traffic(bwd_kernel.split("<")[0])
 
     out = {
         "metric": "fwd+bwd retention TFLOP/s, B=8 H=16 T=4096 d=128 bf16",

@@ -215,12 +215,13 @@ int forward(const Shape& s, const void* q, const void* k, const void* v, const v
   return run(a, stream, "forward");
 }
 
-// The plain backward with dk = dv = 128 has a kernel of its own that reads q, k, v, dO once for dk
+// The plain backward with dk and dv of 64 or 128 has a kernel of its own that reads q, k, v, dO once for dk
 // and dv together (retention_bwd_fused.h); it runs two workgroups per (batch, head) stream, so it
 // is chosen when there are enough streams for the device (below).  The backward choice (FLASHPOP_BWD,
 // fp_set_backward_choice) overrides that (for A/B measurements).
+bool fused_dim(int d) { return d == 64 || d == 128; }
 bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes = false) {
-  if (s.dk != fpk::FB_D || s.dv != fpk::FB_D || d_blocks) return false;
+  if (!fused_dim(s.dk) || !fused_dim(s.dv) || d_blocks) return false;
   if (s.T < 8 * fpk::CH) return false;   // short sequences: the walk over many of them per workgroup serves better
   read_environment();
   const int choice = g_bwd_choice.load(std::memory_order_relaxed);
@@ -274,6 +275,7 @@ int backward_fused(const Shape& s, const void* q, const void* k, const void* v, 
   a.dq = out(dq); a.dk = out(dk_); a.dv = out(dv_);
   a.s0 = in(s0); a.ds_out = in(d_s_out); a.ds0 = out(d_s0);
   a.B = s.B; a.T = s.T; a.H = s.H;
+  a.dk_dim = s.dk; a.dv_dim = s.dv;
   a.scale = 1.0f / std::sqrt((float)s.dk);
   for (int h = 0; h < s.H; ++h) a.log2g[h] = (float)std::log2(decays[h]);
   const char* msg = "";

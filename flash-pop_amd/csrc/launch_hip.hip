@@ -32,26 +32,17 @@ __global__ __launch_bounds__(fpk::NTHREADS_WS) void retention_pass_multi_kernel(
   fpk::retention_pass_ws<DA, MODE, NH>(first, io, lds, id.wg, nwg);
 }
 
+// MODE: how POP suffixes take part (fpk::FbMode): none, as extra stops of the walks, or (at most 16 tokens) folded into
+// the chunks at their boundaries, with suffix_intra_bwd_kernel for what stays inside such a suffix
+template <int DK, int DV, int MODE>
 __global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_kernel(const fpk::FusedBwdArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::fused_bwd<fpk::FB_PLAIN>(args, lds, fprt::block_index());
+  fpk::fused_bwd<DK, DV, MODE>(args, lds, fprt::block_index());
 }
-
-// the same with POP suffixes at the block boundaries, as extra stops of the walks
-__global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_pop_kernel(const fpk::FusedBwdArgs args) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::fused_bwd<fpk::FB_STOPS>(args, lds, fprt::block_index());
-}
-
-// ... with suffixes of at most 16 tokens folded into the chunks at their boundaries, and the kernel for what stays
-// inside such a suffix
-__global__ __launch_bounds__(fpk::FB_THREADS) void retention_bwd_fused_fold_kernel(const fpk::FusedBwdArgs args) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::fused_bwd<fpk::FB_FOLD>(args, lds, fprt::block_index());
-}
+template <int DK, int DV>
 __global__ __launch_bounds__(fpk::SI_THREADS) void suffix_intra_bwd_kernel(const fpk::FusedBwdArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  fpk::suffix_intra_bwd(args, lds);
+  fpk::suffix_intra_bwd<DK, DV>(args, lds);
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -87,7 +78,7 @@ __global__ __launch_bounds__(fpk::LAYER_THREADS) void gated_norm_bwd_kernel(cons
 // launches into a graph after a warm-up run).  Setting the attribute twice in a race is harmless.
 constexpr int kMaxDevices = 64;
 static_assert(2 * fpk::PASS_KERNELS <= 57, "one bit per kernel instantiation, single and paired; the top six for the others");
-std::atomic<uint64_t> g_armed[kMaxDevices];
+std::atomic<uint64_t> g_armed[kMaxDevices][2];   // slots 0..63: pass kernels and the small ones; 64..127: the fused backward family
 
 template <typename Kernel, typename... More>
 int launch(Kernel kernel, int threads, int lds, int slot, int passes, hipStream_t stream, const char** err,
@@ -98,14 +89,14 @@ int launch(Kernel kernel, int threads, int lds, int slot, int passes, hipStream_
     return 1;
   }
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & (1ull << slot))) {
+  if (!tracked || !(g_armed[dev][0].load(std::memory_order_acquire) & (1ull << slot))) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
         hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(1ull << slot, std::memory_order_release);
+    if (tracked) g_armed[dev][0].fetch_or(1ull << slot, std::memory_order_release);
   }
   const int nwg = a.slots * a.H * (a.dB / fpk::BV) * passes;
   hipLaunchKernelGGL(kernel, dim3(nwg), dim3(threads), lds, stream, a, more...);
@@ -226,22 +217,23 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
 
 namespace {
 
-// opts a kernel into `lds` bytes of dynamic LDS once per device (bit `bit` of the per-device word)
+// opts a kernel into `lds` bytes of dynamic LDS once per device (bit `bit` of the 128 per device)
 int arm(const void* kernel, int lds, int bit, const char** err) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     *err = "hipGetDevice failed";
     return 1;
   }
-  const uint64_t mask = 1ull << bit;
+  const uint64_t mask = 1ull << (bit & 63);
+  const int word = bit >> 6;
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & mask)) {
+  if (!tracked || !(g_armed[dev][word].load(std::memory_order_acquire) & mask)) {
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(mask, std::memory_order_release);
+    if (tracked) g_armed[dev][word].fetch_or(mask, std::memory_order_release);
   }
   return 0;
 }
@@ -257,6 +249,40 @@ int launched(const char** err) {
 
 }  // namespace
 
+namespace {
+
+// one (dk, dv) instantiation of the fused backward family; `slot` numbers its four kernels 64 + 4 slot ..
+template <int DK, int DV>
+int launch_bwd_fused(const fpk::FusedBwdArgs& a, int slot, hipStream_t st, const char** err) {
+  const dim3 grid((unsigned)(2 * a.B * a.H)), threads(fpk::FB_THREADS);
+  const int bit = 64 + 4 * slot;
+  if (a.fold) {
+    constexpr int lds = fpk::fb_lds_bytes(DK, DV, fpk::FB_FOLD), lds_si = fpk::si_lds_bytes(DK, DV);
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel<DK, DV, fpk::FB_FOLD>), lds, bit + 2, err)) return 1;
+    if (arm(reinterpret_cast<const void*>(suffix_intra_bwd_kernel<DK, DV>), lds_si, bit + 3, err)) return 1;
+    hipLaunchKernelGGL((retention_bwd_fused_kernel<DK, DV, fpk::FB_FOLD>), grid, threads, lds, st, a);
+    if (launched(err)) return 1;
+    // what stays inside the suffixes, after the part of dq_s that comes from the carried state is written
+    const long long pairs = (long long)a.B * (a.T / a.block + 1) * a.H;
+    const long long wgs = 8LL * fpk_compute_units();
+    hipLaunchKernelGGL((suffix_intra_bwd_kernel<DK, DV>), dim3((unsigned)(pairs < wgs ? pairs : wgs)), dim3(fpk::SI_THREADS),
+                       lds_si, st, a);
+    return launched(err);
+  }
+  if (a.block > 0) {
+    constexpr int lds = fpk::fb_lds_bytes(DK, DV, fpk::FB_STOPS);
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel<DK, DV, fpk::FB_STOPS>), lds, bit + 1, err)) return 1;
+    hipLaunchKernelGGL((retention_bwd_fused_kernel<DK, DV, fpk::FB_STOPS>), grid, threads, lds, st, a);
+  } else {
+    constexpr int lds = fpk::fb_lds_bytes(DK, DV, fpk::FB_PLAIN);
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel<DK, DV, fpk::FB_PLAIN>), lds, bit, err)) return 1;
+    hipLaunchKernelGGL((retention_bwd_fused_kernel<DK, DV, fpk::FB_PLAIN>), grid, threads, lds, st, a);
+  }
+  return launched(err);
+}
+
+}  // namespace
+
 int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char** err) {
   fpk::FusedBwdArgs a = args;
   a.fold = a.block > 0 && a.Ls <= fpk::FB_SFX_ROWS;
@@ -265,27 +291,10 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char
     return 1;
   }
   const hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid((unsigned)(2 * a.B * a.H)), threads(fpk::FB_THREADS);
-  if (a.fold) {
-    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_fold_kernel), fpk::fb_fold_lds_bytes(), 59, err)) return 1;
-    if (arm(reinterpret_cast<const void*>(suffix_intra_bwd_kernel), fpk::si_lds_bytes(), 58, err)) return 1;
-    hipLaunchKernelGGL(retention_bwd_fused_fold_kernel, grid, threads, fpk::fb_fold_lds_bytes(), st, a);
-    if (launched(err)) return 1;
-    // what stays inside the suffixes, after the part of dq_s that comes from the carried state is written
-    const long long pairs = (long long)a.B * (a.T / a.block + 1) * a.H;
-    const long long wgs = 8LL * fpk_compute_units();
-    hipLaunchKernelGGL(suffix_intra_bwd_kernel, dim3((unsigned)(pairs < wgs ? pairs : wgs)), dim3(fpk::SI_THREADS),
-                       fpk::si_lds_bytes(), st, a);
-    return launched(err);
-  }
-  if (a.block > 0) {
-    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_pop_kernel), fpk::fb_lds_bytes(), 62, err)) return 1;
-    hipLaunchKernelGGL(retention_bwd_fused_pop_kernel, grid, threads, fpk::fb_lds_bytes(), st, a);
-  } else {
-    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel), fpk::fb_lds_bytes(), 63, err)) return 1;
-    hipLaunchKernelGGL(retention_bwd_fused_kernel, grid, threads, fpk::fb_lds_bytes(), st, a);
-  }
-  return launched(err);
+  if (a.dk_dim == 128 && a.dv_dim == 128) return launch_bwd_fused<128, 128>(a, 0, st, err);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return launch_bwd_fused<64, 128>(a, 1, st, err);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return launch_bwd_fused<128, 64>(a, 2, st, err);
+  return launch_bwd_fused<64, 64>(a, 3, st, err);
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* stream, const char** err) {
@@ -302,13 +311,13 @@ int fpk_launch_contrib(const fpk::ContribArgs& a, void* stream, const char** err
                                        : reinterpret_cast<const void*>(segment_contrib_kernel<false>);
   const uint64_t bit = 1ull << (a.reverse ? 60 : 61);
   const bool tracked = dev >= 0 && dev < kMaxDevices;
-  if (!tracked || !(g_armed[dev].load(std::memory_order_acquire) & bit)) {
+  if (!tracked || !(g_armed[dev][0].load(std::memory_order_acquire) & bit)) {
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, fpk::sc_lds_bytes()) != hipSuccess) {
       (void)hipGetLastError();
       *err = "hipFuncSetAttribute(MaxDynamicSharedMemorySize) failed";
       return 1;
     }
-    if (tracked) g_armed[dev].fetch_or(bit, std::memory_order_release);
+    if (tracked) g_armed[dev][0].fetch_or(bit, std::memory_order_release);
   }
   const dim3 grid((unsigned)(a.B * a.H * (a.dB / fpk::FB_D))), threads(fpk::FB_THREADS);
   if (a.reverse)

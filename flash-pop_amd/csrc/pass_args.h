@@ -117,14 +117,14 @@ struct DecodeArgs {
   float scale;
   float gamma[MAX_HEADS];
 };
-// The fused backward for dk = dv = 128 (retention_bwd_fused.h): per (batch, head) stream one workgroup
+// The fused backward for dk, dv of 64 or 128 (retention_bwd_fused.h): per (batch, head) stream one workgroup
 // walks backward for dk, dv and d_s0 and one walks forward for dq.
-constexpr int FB_D = 128;
+constexpr int FB_D = 128;                  // the widest head dimension it takes
 constexpr int FB_THREADS = 512;
 struct FusedBwdArgs {
-  const uint16_t *q, *k, *v, *dO;          // [B,T,H,128]
+  const uint16_t *q, *k, *v, *dO;          // q, k [B,T,H,dk_dim]; v, dO [B,T,H,dv_dim]
   uint16_t *dq, *dk, *dv;
-  const uint16_t* s0;                      // [B,H,128,128], nullable (zeros)
+  const uint16_t* s0;                      // [B,H,dk_dim,dv_dim], nullable (zeros)
   const uint16_t* ds_out;                  // gradient of the final state, nullable (zeros)
   uint16_t* ds0;                           // gradient of s0, nullable (not wanted)
   // States that the forward pass left behind every `ckpt_every` tokens (a multiple of 64):
@@ -135,13 +135,14 @@ struct FusedBwdArgs {
   const uint16_t* ckpt;
   int ckpt_every;
   // POP suffixes (block > 0; none of the above checkpoints then): one suffix of Ls <= 64 tokens per
-  // block boundary 0, block, ..., T, tensors [B * (T / block + 1), Ls, H, 128] as in PassArgs; block a
+  // block boundary 0, block, ..., T, tensors [B * (T / block + 1), Ls, H, d] as in PassArgs; block a
   // multiple of 64 that divides T.  A suffix reads the state at its boundary without advancing it.
   const uint16_t *q_sfx, *k_sfx, *v_sfx, *dO_sfx;
   uint16_t *dq_sfx, *dk_sfx, *dv_sfx;
   int block, Ls;
   int fold;                                // suffixes of at most 16 tokens: folded into the chunks at their boundaries (FB_FOLD), set by the launcher
   int B, T, H;
+  int dk_dim, dv_dim;                      // head dimensions: 64 or 128 each
   float scale;                             // dk^-1/2
   float log2g[MAX_HEADS];
 };

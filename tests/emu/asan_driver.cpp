@@ -64,15 +64,15 @@ int pop(int B, int T, int H, int dk, int dv, int block) {
 }
 
 // forward with checkpoints every `every` tokens, then the backward that starts from them
-int checkpointed(int B, int T, int H, int every) {
+int checkpointed(int B, int T, int H, int every, int dk = 128, int dv = 128) {
   std::vector<double> dec(H, 0.97);
-  const int d = 128;
-  const size_t n = (size_t)B * T * H * d, ns = (size_t)B * H * d * d, nc = (size_t)B * (T / every) * H * d * d;
-  uint16_t *q = buf(n), *k = buf(n), *v = buf(n), *s = buf(ns), *o = buf(n, false), *so = buf(ns, false), *ck = buf(nc, false);
-  uint16_t *dO = buf(n), *dS = buf(ns), *dq = buf(n, false), *dk_ = buf(n, false), *dv_ = buf(n, false), *ds0 = buf(ns, false);
-  int rc = fp_retention_fwd_ckpt(q, k, v, s, dec.data(), o, so, ck, every, B, T, H, d, d, nullptr);
-  if (!rc) rc = fp_retention_bwd_ckpt(q, k, v, s, dec.data(), dO, dS, ck, every, dq, dk_, dv_, ds0, B, T, H, d, d, nullptr);
-  return done(rc, "checkpointed", B, T, H, d, d, every);
+  const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv,
+               nc = (size_t)B * (T / every) * H * dk * dv;
+  uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = buf(ns), *o = buf(nv, false), *so = buf(ns, false), *ck = buf(nc, false);
+  uint16_t *dO = buf(nv), *dS = buf(ns), *dq = buf(nq, false), *dk_ = buf(nq, false), *dv_ = buf(nv, false), *ds0 = buf(ns, false);
+  int rc = fp_retention_fwd_ckpt(q, k, v, s, dec.data(), o, so, ck, every, B, T, H, dk, dv, nullptr);
+  if (!rc) rc = fp_retention_bwd_ckpt(q, k, v, s, dec.data(), dO, dS, ck, every, dq, dk_, dv_, ds0, B, T, H, dk, dv, nullptr);
+  return done(rc, "checkpointed", B, T, H, dk, dv, every);
 }
 
 // nblk full blocks and `tail` < block tokens after them
@@ -147,6 +147,11 @@ int main() {
   rc |= fused(1, 8, 64, 16, 1, 128, 128);     // backward in the kernel that carries dS once, suffixes as extra stops
   rc |= plain(1, 530, 1, 128, 128, false);    // the same kernel without suffixes, ragged last chunk
   rc |= checkpointed(1, 600, 1, 128);         // ... with the forward's checkpoints
+  rc |= fused(1, 8, 64, 16, 1, 64, 128);      // the same kernels for 64-wide keys: folded suffixes,
+  rc |= fused(1, 4, 128, 40, 1, 128, 64);     // 64-wide values with the suffixes as stops,
+  rc |= plain(1, 530, 1, 64, 64, false);      // 64 x 64 states (half of the waves own a tile), ragged last chunk,
+  rc |= checkpointed(1, 600, 1, 256, 64, 128);   // checkpoints of 64 x 128 states
+  rc |= fused(1, 8, 64, 9, 1, 64, 64);        // folded suffixes of 9 tokens on 64 x 64 states
   fp_set_backward_choice(0, -1);
   rc |= decode(2, 3, 64, 128);
   rc |= decode(1, 1, 256, 256);

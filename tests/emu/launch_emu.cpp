@@ -71,6 +71,26 @@ int fpk_stream_is_capturing(void* /*stream*/) { return g_emu_capturing; }
 // ones take on a real device (several sequences per workgroup, split sequences).
 int fpk_compute_units() { return 8; }
 
+namespace {
+
+template <int DK, int DV>
+int emu_bwd_fused(const fpk::FusedBwdArgs& a) {
+  if (a.fold) {
+    if (int rc = run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_FOLD),
+                          [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_FOLD>(a, l, fprt::block_index()); }))
+      return rc;
+    const int pairs = a.B * (a.T / a.block + 1) * a.H;
+    return run_grid(fpk::SI_THREADS, pairs < 3 ? pairs : 3, fpk::si_lds_bytes(DK, DV), [&](char* l) { fpk::suffix_intra_bwd<DK, DV>(a, l); });
+  }
+  if (a.block > 0)
+    return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_STOPS),
+                    [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_STOPS>(a, l, fprt::block_index()); });
+  return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_PLAIN),
+                  [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_PLAIN>(a, l, fprt::block_index()); });
+}
+
+}  // namespace
+
 int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const char** err) {
   fpk::FusedBwdArgs a = args;
   a.fold = a.block > 0 && a.Ls <= fpk::FB_SFX_ROWS;
@@ -78,17 +98,10 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const 
     *err = why;
     return 1;
   }
-  if (a.fold) {
-    if (int rc = run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_fold_lds_bytes(),
-                          [&](char* l) { fpk::fused_bwd<fpk::FB_FOLD>(a, l, fprt::block_index()); }))
-      return rc;
-    const int pairs = a.B * (a.T / a.block + 1) * a.H;
-    return run_grid(fpk::SI_THREADS, pairs < 3 ? pairs : 3, fpk::si_lds_bytes(), [&](char* l) { fpk::suffix_intra_bwd(a, l); });
-  }
-  return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(), [&](char* l) {
-    if (a.block > 0) fpk::fused_bwd<fpk::FB_STOPS>(a, l, fprt::block_index());
-    else fpk::fused_bwd<fpk::FB_PLAIN>(a, l, fprt::block_index());
-  });
+  if (a.dk_dim == 128 && a.dv_dim == 128) return emu_bwd_fused<128, 128>(a);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return emu_bwd_fused<64, 128>(a);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return emu_bwd_fused<128, 64>(a);
+  return emu_bwd_fused<64, 64>(a);
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* /*stream*/, const char** err) {

@@ -139,47 +139,57 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
     assert torch.equal(o2, o) and all(torch.equal(a, b) for a, b in zip(again, (dq, dk_, dv_, ds0)))
 
 
-@pytest.mark.parametrize("B,nblk,block,Ls,H,state_std", [
-    (1, 4, 128, 16, 1, 0.5),     # two chunks per block
-    (1, 8, 64, 64, 1, None),     # block == chunk, suffixes as long as a chunk, no initial state
-    (1, 3, 192, 1, 2, 0.3),      # three chunks per block, one-token suffixes, two heads
-    (1, 8, 64, 9, 1, 0.3),       # short suffixes folded into every chunk; 9 suffixes over 3 workgroups of the second kernel
+@pytest.mark.parametrize("B,nblk,block,Ls,H,state_std,dk,dv", [
+    (1, 4, 128, 16, 1, 0.5, 128, 128),     # two chunks per block
+    (1, 8, 64, 64, 1, None, 128, 128),     # block == chunk, suffixes as long as a chunk, no initial state
+    (1, 3, 192, 1, 2, 0.3, 128, 128),      # three chunks per block, one-token suffixes, two heads
+    (1, 8, 64, 9, 1, 0.3, 128, 128),       # short suffixes folded into every chunk; 9 suffixes over 3 workgroups of the second kernel
+    (1, 8, 64, 16, 2, 0.3, 64, 128),       # 64-wide keys: folded suffixes
+    (1, 4, 128, 40, 1, None, 128, 64),     # 64-wide values: suffixes as stops, no initial state
+    (1, 8, 64, 9, 1, 0.5, 64, 64),         # 64 x 64 states: four state tiles for eight waves
 ])
-def test_fused_pop_backward_that_carries_ds_once(emu_lib, choose_backward, B, nblk, block, Ls, H, state_std):
-    """dk = dv = 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
+def test_fused_pop_backward_that_carries_ds_once(emu_lib, choose_backward, B, nblk, block, Ls, H, state_std, dk, dv):
+    """dk, dv of 64 or 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
     the kernel that walks backward once for dk and dv beside a forward walk for dq, with the
-    suffixes as extra stops at the block boundaries.  Same results as the pass-per-gradient path."""
+    suffixes as extra stops at the block boundaries or folded into the chunks there.  Same results as the
+    pass-per-gradient path."""
     decays = oracle.head_decays(H, (4, 9))
     T = nblk * block
-    q, k, v, s = hp.make_inputs(B, T, H, 128, 128, seed=T + Ls, state_std=state_std)
-    sfx = hp.make_suffix_inputs(B, nblk, Ls, H, 128, 128, seed=T + Ls + 1)
-    cot = hp.make_cotangents([(B, T, H, 128), tuple(sfx[2].shape), (B, H, 128, 128)], seed=T + 2)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + Ls, state_std=state_std)
+    sfx = hp.make_suffix_inputs(B, nblk, Ls, H, dk, dv, seed=T + Ls + 1)
+    cot = hp.make_cotangents([(B, T, H, dv), tuple(sfx[2].shape), (B, H, dk, dv)], seed=T + 2)
     choose_backward(FUSED)
     grads = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
     _, _, _, g_ref = hp.oracle_fused(q, k, v, s, sfx, decays, block, cot)
     _check_all([(n, g, r) for n, g, r in zip(FUSED_NAMES, grads, g_ref)])
     choose_backward(PASSES)
     other = hp.raw_fused_bwd(emu_lib, q, k, v, s, sfx, decays, block, cot)
+    differs = False
     for name, x, y in zip(FUSED_NAMES, grads, other):
         if x is not None:
             assert hp.error_report(x, y.float())["rms_ratio"] < 0.004, name
+            differs = differs or not torch.equal(x, y)
+    assert differs, "the forced choice made no difference: both calls took the same kernels"
 
 
-@pytest.mark.parametrize("B,T,H,state_std,every", [
-    (1, 700, 1, 0.5, 128),      # ragged tail beyond the last checkpoint, initial state
-    (1, 512, 1, None, 256),     # the sequence ends on a checkpoint, no initial state
-    (2, 520, 1, 0.3, 64),       # a checkpoint after every chunk, two sequences
-    (1, 600, 1, 0.2, 1024),     # interval longer than the sequence: no checkpoint at all
-    (1, 576, 1, 0.4, 0),        # no checkpoint buffer: the fused backward walks forward from s0
+@pytest.mark.parametrize("B,T,H,state_std,every,dk,dv", [
+    (1, 700, 1, 0.5, 128, 128, 128),      # ragged tail beyond the last checkpoint, initial state
+    (1, 512, 1, None, 256, 128, 128),     # the sequence ends on a checkpoint, no initial state
+    (2, 520, 1, 0.3, 64, 128, 128),       # a checkpoint after every chunk, two sequences
+    (1, 600, 1, 0.2, 1024, 128, 128),     # interval longer than the sequence: no checkpoint at all
+    (1, 576, 1, 0.4, 0, 128, 128),        # no checkpoint buffer: the fused backward walks forward from s0
+    (1, 700, 2, 0.5, 256, 64, 128),       # 64-wide keys
+    (1, 530, 1, None, 0, 128, 64),        # 64-wide values, no checkpoints, no initial state
+    (1, 600, 1, 0.3, 128, 64, 64),        # 64 x 64 states
 ])
-def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, state_std, every):
-    """dk = dv = 128 and at least eight chunks: the backward that carries dS once, beside the
+def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, state_std, every, dk, dv):
+    """dk, dv of 64 or 128 and at least eight chunks: the backward that carries dS once, beside the
     workgroup that re-runs the state from the checkpoints the forward left (segments taken from
     the last to the first)."""
     choose_backward(FUSED)
     decays = oracle.head_decays(H)
-    q, k, v, s = hp.make_inputs(B, T, H, 128, 128, seed=T, state_std=state_std)
-    d_o, d_s = hp.make_cotangents([(B, T, H, 128), (B, H, 128, 128)], seed=T + 1)
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T, state_std=state_std)
+    d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=T + 1)
     if every:
         o, S, dq, dk_, dv_, ds0 = hp.raw_ckpt_fwd_bwd(emu_lib, q, k, v, s, decays, d_o, d_s, every)
     else:
@@ -193,6 +203,10 @@ def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, stat
     assert torch.equal(o, o2) and torch.equal(S, S2)
     assert torch.equal(dk_, g2[1]) and torch.equal(dv_, g2[2])
     assert (ds0 is None and g2[3] is None) or torch.equal(ds0, g2[3])
+    # and the pass-per-gradient backward gives other bits: the forced choice is what ran
+    choose_backward(PASSES)
+    g3 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
+    assert not torch.equal(g3[1], dk_)
 
 
 def test_c_entry_points_refuse_a_capturing_stream(emu_lib):
@@ -240,7 +254,8 @@ def test_checkpoint_size_query(emu_lib, choose_backward):
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 2 * 2 * (4096 // 512) * 4 * 128 * 128
     assert every.value == 512
     assert emu_lib.fp_retention_checkpoint_bytes(2, 512, 4, 128, 128, ctypes.byref(every)) == 0 and every.value == 0
-    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 64, 128, ctypes.byref(every)) == 0
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 64, 128, ctypes.byref(every)) == 2 * 2 * (4096 // 512) * 4 * 64 * 128
+    assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 64, 256, ctypes.byref(every)) == 0
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, None) > 0
     choose_backward(PASSES)
     assert emu_lib.fp_retention_checkpoint_bytes(2, 4096, 4, 128, 128, ctypes.byref(every)) == 0

@@ -68,6 +68,9 @@ def run_fused(B, N, block, Ls, H, dk, dv, state_std, seed, decay_range=None, ora
     (1, 2, 96, 24, 2, 128, 256),     # 256-wide values: two visits per chunk in the dq and dk passes
     (2, 3, 64, 16, 2, 192, 192),     # 192-wide keys and values: three visits per chunk in every pass
     (3, 8, 64, 16, 16, 128, 128),    # 48 streams: the fewest that take the backward with the suffixes folded into the chunks
+    (8, 8, 64, 16, 12, 64, 128),     # ... the same backward for 64-wide keys (96 streams)
+    (4, 4, 128, 40, 12, 128, 64),    # ... 64-wide values, suffixes as extra stops of the walks
+    (8, 8, 64, 9, 8, 64, 64),        # ... 64 x 64 states, folded suffixes of 9 tokens
     (3, 4, 128, 33, 16, 128, 128),   # ... with suffixes too long to fold: stops of its walks
 ])
 def test_fused_parity_sweep(B, N, block, Ls, H, dk, dv):

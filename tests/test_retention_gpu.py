@@ -65,9 +65,27 @@ def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, 
     (6, 1000, 16, 128, 128, 0.1),    # the backward that carries dS once, one checkpoint and a ragged stretch after it
     (3, 513, 32, 128, 128, None),    # ... a one-token last chunk behind the only checkpoint, no state argument
     (2, 2100, 64, 128, 128, 0.05),   # ... four checkpoints, 64 heads
+    (8, 1100, 12, 64, 128, 0.05),    # the same kernel for 64-wide keys (96 streams), two checkpoints and a ragged stretch
+    (6, 700, 16, 128, 64, None),     # ... 64-wide values, one checkpoint, no state argument
+    (11, 577, 8, 64, 64, 0.1),       # ... 64 x 64 states (half of the waves own a state tile), one-token last chunk
 ])
 def test_parity_sweep(B, T, H, dk, dv, state_std):
     run_plain(B, T, H, dk, dv, state_std, seed=T + dk)
+
+
+@pytest.mark.parametrize("choice,B,T,H,dk,dv", [
+    (2, 2, 1024, 4, 128, 128),    # the fused backward forced where the shape alone would take the passes (8 streams)
+    (2, 1, 640, 3, 64, 128),
+    (1, 8, 1024, 16, 128, 128),   # the passes forced where the shape alone would take the fused backward (128 streams)
+    (1, 8, 640, 12, 64, 128),
+])
+def test_forced_backward_choice(hip_lib, choice, B, T, H, dk, dv):
+    """fp_set_backward_choice: both backward paths of a shape against the oracle, whatever the library would pick."""
+    assert hip_lib.fp_set_backward_choice(choice, -1) == 0
+    try:
+        run_plain(B, T, H, dk, dv, 0.1, seed=T + choice)
+    finally:
+        assert hip_lib.fp_set_backward_choice(0, -1) == 0
 
 
 def test_decay_range_of_reference_tests():
