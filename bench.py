@@ -10,7 +10,7 @@ the CPU oracle timed on the host cores beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--spin-up S] [--no-cpu] [--no-pop] [--no-long]
                     [--no-layer5] [--no-layer] [--no-model]
-    python bench.py --profile-leg {headline,pop_fused,pop_two_op,long,layer5} --steps K
+    python bench.py --profile-leg {headline,pop_fused,pop_two_op,long,layer5,layer_ops} --steps K
         exactly K steps of one workload and nothing else: what the rocprofv3 runs of profile_counters.sh trace
 """
 import argparse
@@ -214,7 +214,28 @@ def workload_long(dev):
                   "flops": algorithmic_flops(B, T, H, dk, dv)}
 
 
-WORKLOADS = {"headline": workload_headline, "pop_fused": workload_pop_fused, "pop_two_op": workload_pop_two_op,
+def workload_layer_ops(dev):
+    """The two elementwise stages around the op at config 2's tensor shapes: rotary embedding of q and k, per-head
+    norm + swish gate forward and backward, one launch each."""
+    import torch
+    from flash_pop_amd import XPos, gated_group_norm
+    B, T, H, d = 8, 4096, 16, 128
+    g = torch.Generator(device=dev).manual_seed(7)
+    q, k, r, gate, d_out = (torch.randn(B, T, H, d, generator=g, device=dev).to(torch.bfloat16) for _ in range(5))
+    gate, d_out = gate.flatten(-2), d_out.flatten(-2)
+    xpos = XPos(d)
+    rl, gl = r.requires_grad_(), gate.requires_grad_()
+
+    def step(ev=None):
+        xpos(q, k, 0)
+        out = gated_group_norm(rl, gl, 1e-6)
+        torch.autograd.grad(out, [rl, gl], d_out)
+
+    n = q.numel() * 2
+    return step, {"shape": (B, T, H, d, d), "tokens": B * T, "bytes": (7 * n, 5 * n)}
+
+
+WORKLOADS = {"headline": workload_headline, "layer_ops": workload_layer_ops, "pop_fused": workload_pop_fused, "pop_two_op": workload_pop_two_op,
              "long": workload_long, "layer5": workload_layer5}
 
 

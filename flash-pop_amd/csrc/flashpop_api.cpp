@@ -220,8 +220,11 @@ int forward(const Shape& s, const void* q, const void* k, const void* v, const v
 // is chosen when there are enough streams for the device (below).  The backward choice (FLASHPOP_BWD,
 // fp_set_backward_choice) overrides that (for A/B measurements).
 bool fused_dim(int d) { return d == 64 || d == 128; }
-bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes = false) {
-  if (!fused_dim(s.dk) || !fused_dim(s.dv) || d_blocks) return false;
+// `d_blocks` with `block`: gradients of POP block states arrive; the kernel adds them on its way when the blocks are
+// whole chunks.
+bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes = false, int block = 0) {
+  if (!fused_dim(s.dk) || !fused_dim(s.dv)) return false;
+  if (d_blocks && (block <= 0 || block % fpk::CH != 0)) return false;
   if (s.T < 8 * fpk::CH) return false;   // short sequences: the walk over many of them per workgroup serves better
   read_environment();
   const int choice = g_bwd_choice.load(std::memory_order_relaxed);
@@ -260,9 +263,11 @@ struct SuffixGrads {
 int backward_fused(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
                    const void* d_o, const void* d_s_out, void* dq, void* dk_, void* dv_, void* d_s0, void* stream,
                    const void* ckpt = nullptr, int ckpt_every = 0, const Suffixes* sfx = nullptr,
-                   const SuffixGrads* sg = nullptr) {
+                   const SuffixGrads* sg = nullptr, const void* d_blocks = nullptr, int blocks_every = 0) {
   fpk::FusedBwdArgs a;
   std::memset(&a, 0, sizeof a);
+  a.d_blocks = in(d_blocks);
+  a.blocks_every = d_blocks ? blocks_every : 0;
   a.ckpt = in(ckpt);
   a.ckpt_every = ckpt ? ckpt_every : 0;
   if (sfx) {
@@ -283,10 +288,38 @@ int backward_fused(const Shape& s, const void* q, const void* k, const void* v, 
   return FP_OK;
 }
 
+// Many short sequences that each read a state of their own and whose final states nobody differentiates (the
+// suffix call of the reference's POP layer): one kernel that takes a (sequence, head) pair per step (short_seq.h)
+// instead of a 64-token item per pass and pair.
+bool use_short_backward(const Shape& s, const void* d_s_out, const void* d_blocks) {
+  if (s.T > fpk::SS_ROWS || d_s_out || d_blocks || !fused_dim(s.dk) || !fused_dim(s.dv)) return false;
+  read_environment();
+  return g_bwd_choice.load(std::memory_order_relaxed) != BWD_PASSES;
+}
+
+int backward_short(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
+                   const void* d_o, void* dq, void* dk_, void* dv_, void* d_s0, void* stream) {
+  fpk::FusedBwdArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.q = in(q); a.k = in(k); a.v = in(v); a.dO = in(d_o);
+  a.dq = out(dq); a.dk = out(dk_); a.dv = out(dv_);
+  a.s0 = in(s0); a.ds0 = out(d_s0);
+  a.B = s.B; a.T = s.T; a.H = s.H;
+  a.dk_dim = s.dk; a.dv_dim = s.dv;
+  a.scale = 1.0f / std::sqrt((float)s.dk);
+  for (int h = 0; h < s.H; ++h) a.log2g[h] = (float)std::log2(decays[h]);
+  const char* msg = "";
+  if (fpk_launch_short_bwd(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "short-sequence backward: %s", msg);
+  return FP_OK;
+}
+
 int backward(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays,
              const void* d_o, const void* d_s_out, const void* d_blocks, int block, void* dq, void* dk_, void* dv_,
              void* d_s0, void* stream) {
-  if (use_fused_backward(s, d_blocks)) return backward_fused(s, q, k, v, s0, decays, d_o, d_s_out, dq, dk_, dv_, d_s0, stream);
+  if (use_short_backward(s, d_s_out, d_blocks)) return backward_short(s, q, k, v, s0, decays, d_o, dq, dk_, dv_, d_s0, stream);
+  if (use_fused_backward(s, d_blocks, false, block) && !(d_blocks && d_s_out))
+    return backward_fused(s, q, k, v, s0, decays, d_o, d_s_out, dq, dk_, dv_, d_s0, stream, nullptr, 0, nullptr, nullptr,
+                          d_blocks, block);
   const float sc = 1.0f / std::sqrt((float)s.dk);
   const int nblk = block > 0 ? s.T / block : 0;
   fpk::PassArgs g, a;

@@ -6,6 +6,7 @@
 #include "segment_scan.h"
 #include "segment_contrib.h"
 #include "retention_bwd_fused.h"
+#include "short_seq.h"
 #include "decode_step.h"
 #include "layer_ops.h"
 
@@ -43,6 +44,12 @@ template <int DK, int DV>
 __global__ __launch_bounds__(fpk::SI_THREADS) void suffix_intra_bwd_kernel(const fpk::FusedBwdArgs args) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   fpk::suffix_intra_bwd<DK, DV>(args, lds);
+}
+
+template <int DK, int DV>
+__global__ __launch_bounds__(fpk::FB_THREADS) void short_seq_bwd_kernel(const fpk::FusedBwdArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::short_seq_bwd<DK, DV>(args, lds);
 }
 
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
@@ -251,11 +258,17 @@ int launched(const char** err) {
 
 namespace {
 
-// one (dk, dv) instantiation of the fused backward family; `slot` numbers its four kernels 64 + 4 slot ..
+// one (dk, dv) instantiation of the fused backward family; `slot` numbers its five kernels 64 + 5 slot ..
 template <int DK, int DV>
 int launch_bwd_fused(const fpk::FusedBwdArgs& a, int slot, hipStream_t st, const char** err) {
   const dim3 grid((unsigned)(2 * a.B * a.H)), threads(fpk::FB_THREADS);
-  const int bit = 64 + 4 * slot;
+  const int bit = 64 + 5 * slot;
+  if (a.d_blocks) {
+    constexpr int lds = fpk::fb_lds_bytes(DK, DV, fpk::FB_BLOCKS);
+    if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel<DK, DV, fpk::FB_BLOCKS>), lds, bit + 4, err)) return 1;
+    hipLaunchKernelGGL((retention_bwd_fused_kernel<DK, DV, fpk::FB_BLOCKS>), grid, threads, lds, st, a);
+    return launched(err);
+  }
   if (a.fold) {
     constexpr int lds = fpk::fb_lds_bytes(DK, DV, fpk::FB_FOLD), lds_si = fpk::si_lds_bytes(DK, DV);
     if (arm(reinterpret_cast<const void*>(retention_bwd_fused_kernel<DK, DV, fpk::FB_FOLD>), lds, bit + 2, err)) return 1;
@@ -295,6 +308,31 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char
   if (a.dk_dim == 64 && a.dv_dim == 128) return launch_bwd_fused<64, 128>(a, 1, st, err);
   if (a.dk_dim == 128 && a.dv_dim == 64) return launch_bwd_fused<128, 64>(a, 2, st, err);
   return launch_bwd_fused<64, 64>(a, 3, st, err);
+}
+
+namespace {
+
+template <int DK, int DV>
+int launch_short_bwd(const fpk::FusedBwdArgs& a, int slot, hipStream_t st, const char** err) {
+  constexpr int lds = fpk::ss_lds_bytes(DK, DV);
+  if (arm(reinterpret_cast<const void*>(short_seq_bwd_kernel<DK, DV>), lds, 64 + 20 + slot, err)) return 1;
+  const long long pairs = (long long)a.B * a.H, wgs = fpk_compute_units();   // one workgroup per unit: its LDS fills it
+  hipLaunchKernelGGL((short_seq_bwd_kernel<DK, DV>), dim3((unsigned)(pairs < wgs ? pairs : wgs)), dim3(fpk::FB_THREADS), lds, st, a);
+  return launched(err);
+}
+
+}  // namespace
+
+int fpk_launch_short_bwd(const fpk::FusedBwdArgs& a, void* stream, const char** err) {
+  if (const char* why = fpk::check_short_seq_bwd(a)) {
+    *err = why;
+    return 1;
+  }
+  const hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a.dk_dim == 128 && a.dv_dim == 128) return launch_short_bwd<128, 128>(a, 0, st, err);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return launch_short_bwd<64, 128>(a, 1, st, err);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return launch_short_bwd<128, 64>(a, 2, st, err);
+  return launch_short_bwd<64, 64>(a, 3, st, err);
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* stream, const char** err) {

@@ -121,6 +121,8 @@ struct DecodeArgs {
 // walks backward for dk, dv and d_s0 and one walks forward for dq.
 constexpr int FB_D = 128;                  // the widest head dimension it takes
 constexpr int FB_THREADS = 512;
+constexpr int SS_ROWS = 32;                // longest sequence of the backward for many short sequences (short_seq.h), which takes
+                                           // the same arguments: q .. dv, s0, ds0, B, T, H, the head dimensions, scale, log2g
 struct FusedBwdArgs {
   const uint16_t *q, *k, *v, *dO;          // q, k [B,T,H,dk_dim]; v, dO [B,T,H,dv_dim]
   uint16_t *dq, *dk, *dv;
@@ -141,6 +143,11 @@ struct FusedBwdArgs {
   uint16_t *dq_sfx, *dk_sfx, *dv_sfx;
   int block, Ls;
   int fold;                                // suffixes of at most 16 tokens: folded into the chunks at their boundaries (FB_FOLD), set by the launcher
+  // POP block states (no suffixes, no checkpoints then): d_blocks[b][m][h] is the gradient of the state after token
+  // (m + 1) * blocks_every - 1, m < T / blocks_every; blocks_every a multiple of 64.  The reverse walk adds it to dS
+  // where it crosses that boundary.
+  const uint16_t* d_blocks;
+  int blocks_every;
   int B, T, H;
   int dk_dim, dv_dim;                      // head dimensions: 64 or 128 each
   float scale;                             // dk^-1/2
@@ -202,6 +209,9 @@ int fpk_launch_passes(const fpk::PassArgs* const* passes, int n, void* stream, c
 
 // Launches the fused backward (2 B H workgroups).  Same conventions as fpk_launch_pass.
 int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char** err);
+
+// Launches the backward for many short sequences (short_seq.h: T <= 32, no gradient of the final state).
+int fpk_launch_short_bwd(const fpk::FusedBwdArgs& args, void* stream, const char** err);
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);

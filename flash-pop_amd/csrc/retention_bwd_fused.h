@@ -72,7 +72,9 @@ constexpr int FB_XP = 32 * 32;              // elements of one score tile in ope
 //             the chunk's own read-out and writes that part of dq_s); what stays inside a suffix (dk_s, dv_s and the
 //             rest of dq_s) is the work of suffix_intra_bwd, which runs afterwards.  Both walks take one more, empty,
 //             chunk at T for the suffix there.
-enum FbMode { FB_PLAIN = 0, FB_STOPS = 1, FB_FOLD = 2 };
+//   FB_BLOCKS no suffixes, but gradients of the states at block boundaries (the POP operator's block states) join dS
+//             on the way: the reverse workgroup adds d_blocks[m] when its walk crosses the boundary behind block m
+enum FbMode { FB_PLAIN = 0, FB_STOPS = 1, FB_FOLD = 2, FB_BLOCKS = 3 };
 constexpr int FB_SFX_ROWS = 16;                         // longest suffix of FB_FOLD
 // LDS of a launch (the larger of its two kinds of workgroup), bytes.
 //   reverse: q, dO, k, v tiles; bf16 copy of dS; staging tiles for dv and dk; six score tiles;
@@ -388,7 +390,8 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   using GK = FbTile<DK>;
   using GV = FbTile<DV>;
   constexpr int LDK = GK::LD, LDV = GV::LD;
-  constexpr bool SFX = MODE == FB_STOPS, FOLD = MODE == FB_FOLD;
+  constexpr bool SFX = MODE == FB_STOPS, FOLD = MODE == FB_FOLD, BLOCKS = MODE == FB_BLOCKS;
+  static_assert(CH * (LDK + LDV) >= DK * LDV, "a block state's gradient fits where the k and v tiles are");
   const Common k = make_common(p, stream);
   uint16_t* const Qs = reinterpret_cast<uint16_t*>(lds);   // q  [64][LDK]
   uint16_t* const Gs = Qs + GK::ELEMS;                     // dO [64][LDV]
@@ -464,6 +467,13 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     if (sfx_q) st128(QS + at<LDK>(sfx_row, 8 * sfx_piece), v);
     else st128(GS + at<LDV>(sfx_row, 8 * sfx_piece), v);
   };
+  // BLOCKS: the gradient of the block state at token t0 > 0 (the state that the chunk before t0 leaves), or nullptr
+  const int nblocks = BLOCKS ? k.T / p.blocks_every : 0;
+  auto block_grad = [&](int t0) -> const uint16_t* {
+    if (!BLOCKS || t0 <= 0 || t0 % p.blocks_every != 0 || t0 / p.blocks_every > nblocks) return nullptr;
+    return p.d_blocks + (((size_t)k.b * nblocks + (t0 / p.blocks_every - 1)) * p.H + k.h) * DK * DV;
+  };
+  constexpr int BP = DK * (DV / 8) / FB_THREADS;   // 16-byte pieces of a state matrix per thread
   Item cur = item_of(0), nxt = item_of(1), prev = cur;
   u32x4 pf_q[GK::NU], pf_g[GV::NU], pf_k[GK::NU], pf_v[GV::NU], pf_s = {0, 0, 0, 0};
   load_tile<DK, true>(k, p.q, p.q_sfx, cur, pf_q);   // q: read by this workgroup only
@@ -471,7 +481,8 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
   load_tile<DK>(k, p.k, p.k_sfx, cur, pf_k);
   load_tile<DV>(k, p.v, p.v_sfx, cur, pf_v);
   if constexpr (FOLD) pf_s = load_suffix(0);
-  load_state<DK, DV, false>(k, Rt, p.ds_out ? p.ds_out + (size_t)stream * DK * DV : nullptr);
+  // the gradient that the walk starts from: that of the final state, or (BLOCKS) of a block that ends with the sequence
+  load_state<DK, DV, false>(k, Rt, BLOCKS ? block_grad(k.T) : p.ds_out ? p.ds_out + (size_t)stream * DK * DV : nullptr);
   stage_tile<DK>(k, Qs, pf_q);
   stage_tile<DV>(k, Gs, pf_g);
   stage_tile<DK>(k, Ks, pf_k);
@@ -567,6 +578,9 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
 
     // FOLD: the next chunk's suffix rows travel during this stretch only (registers are scarce in the first one)
     if constexpr (FOLD) pf_s = load_suffix(it + 1);
+    // BLOCKS: this chunk starts at a block boundary: the gradient of the state there travels during this stretch
+    const uint16_t* const inject = BLOCKS && !cur.sfx && L > 0 ? block_grad((int)(cur.row - (uint32_t)k.b * k.T)) : nullptr;
+    u32x4 pf_b[BP];
     // ---- stretch 2: Y^T[n][i] += sum_j Z^T[n][j] P^T[j][i]
     if (has_out) {
       u32x4 za[4], pq0[4], pq1[2];
@@ -582,6 +596,11 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
         acc[0] = fprt::mfma_32x32x16_bf16(za[tj], pq0[tj], acc[0]);
         if (tj >= 2) acc[1] = fprt::mfma_32x32x16_bf16(za[tj], pq1[tj - 2], acc[1]);
       }
+    }
+    if constexpr (BLOCKS) {
+      const fprt::BufView bv = fprt::make_buf(inject, inject ? (uint32_t)(DK * DV * 2) : 0u);
+#pragma unroll
+      for (int u = 0; u < BP; ++u) pf_b[u] = fprt::buf_load128(bv, (uint32_t)(k.tid + FB_THREADS * u) * 16);
     }
     // state update, dS[a][n] = gamma^L dS + sum_j gamma^(j+1) q[j][a] dO[j][n], operands two k-steps ahead
     {
@@ -639,10 +658,30 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
       }
     }
     // nobody reads this chunk's k and v tiles or the old copy of dS any more
-    stage_tile<DK>(k, Ks, pf_k);
-    stage_tile<DV>(k, Vs, pf_v);
-    load_tile<DK>(k, p.k, p.k_sfx, after, pf_k);
-    load_tile<DV>(k, p.v, p.v_sfx, after, pf_v);
+    if (BLOCKS && inject) {
+      // the block state's gradient takes the place of the k and v tiles, [dk][dv] as it is stored, and every wave
+      // adds its tiles of it to dS; the next chunk's k and v tiles follow in the third stretch
+      uint16_t* const Bt = Ks;
+#pragma unroll
+      for (int u = 0; u < BP; ++u) {
+        const int pc = k.tid + FB_THREADS * u;
+        st128(Bt + at<LDV>(pc / (DV / 8), 8 * (pc % (DV / 8))), pf_b[u]);
+      }
+      fprt::block_sync();
+      if (owns) {
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            racc[u][r] += bf16_bits_to_float(reinterpret_cast<const u16_m*>(Bt)[at<LDV>(32 * at_ + acc_row(r, g), 32 * (nt0 + u) + c)]);
+        }
+      }
+    } else {
+      stage_tile<DK>(k, Ks, pf_k);
+      stage_tile<DV>(k, Vs, pf_v);
+      load_tile<DK>(k, p.k, p.k_sfx, after, pf_k);
+      load_tile<DV>(k, p.v, p.v_sfx, after, pf_v);
+    }
     if (owns) {
 #pragma unroll
       for (int u = 0; u < TPW; ++u) put_state<LDK>(Rt, 32 * (nt0 + u) + c, 32 * at_, g, racc[u]);
@@ -650,6 +689,12 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     fprt::block_sync();
 
     // ---- stretch 3: every read of this chunk's q and dO tiles is done
+    if (BLOCKS && inject) {
+      stage_tile<DK>(k, Ks, pf_k);
+      stage_tile<DV>(k, Vs, pf_v);
+      load_tile<DK>(k, p.k, p.k_sfx, after, pf_k);
+      load_tile<DV>(k, p.v, p.v_sfx, after, pf_v);
+    }
     stage_tile<DK>(k, Qs, pf_q);
     stage_tile<DV>(k, Gs, pf_g);
     load_tile<DK, true>(k, p.q, p.q_sfx, after, pf_q);
@@ -978,8 +1023,8 @@ FP_DEVICE void fused_bwd(const FusedBwdArgs& p, char* lds, int block) {
     if (fprt::thread_index() < 256) fused_bwd_reverse<DK, DV, 0, MODE>(p, lds, block);
     else fused_bwd_reverse<DK, DV, 1, MODE>(p, lds, block);
   }
-  else if (fprt::thread_index() < 256) fused_bwd_forward<DK, DV, false, MODE>(p, lds, block - streams);
-  else fused_bwd_forward<DK, DV, true, MODE>(p, lds, block - streams);
+  else if (fprt::thread_index() < 256) fused_bwd_forward<DK, DV, false, MODE == FB_BLOCKS ? FB_PLAIN : MODE>(p, lds, block - streams);
+  else fused_bwd_forward<DK, DV, true, MODE == FB_BLOCKS ? FB_PLAIN : MODE>(p, lds, block - streams);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1127,8 +1172,10 @@ inline const char* check_fused_bwd(const FusedBwdArgs& a) {
       !a.dO || !a.dq || !a.dk || !a.dv)
     return "fused backward: bad arguments";
   if (!fused_bwd_dims(a.dk_dim, a.dv_dim)) return "fused backward: dk and dv of 64 or 128";
-  if (a.ckpt && (a.ckpt_every <= 0 || a.ckpt_every % CH != 0 || a.block > 0))
-    return "fused backward: checkpoints every positive multiple of 64 tokens, and not together with suffixes";
+  if (a.ckpt && (a.ckpt_every <= 0 || a.ckpt_every % CH != 0 || a.block > 0 || a.d_blocks))
+    return "fused backward: checkpoints every positive multiple of 64 tokens, and not together with suffixes or block states";
+  if (a.d_blocks && (a.blocks_every <= 0 || a.blocks_every % CH != 0 || a.block > 0 || a.ds_out))
+    return "fused backward with block-state gradients: blocks of a positive multiple of 64 tokens, no suffixes, no final-state gradient";
   if (a.block > 0) {
     if (a.block % CH != 0 || a.T % a.block != 0 || a.Ls < 1 || a.Ls > CH)
       return "fused backward with suffixes: block a multiple of 64 that divides T, 1 <= Ls <= 64";

@@ -5,14 +5,14 @@
 # per run, no spin-up, so that a run holds exactly K steps), then the same HBM counters on a plain copy of
 # known size for scaling, then a kernel trace of the model-level run.  Raw output goes to the directory given
 # as the first argument; profile_summary.py turns it into the tables kept under profiles/.
-#   usage: ./profile_counters.sh <output directory> [workloads, default: all five]
+#   usage: ./profile_counters.sh <output directory> [workloads, default: all]
 set -e
 R=$(cd "$(dirname "$0")" && pwd)
-[ -n "$1" ] || { echo "usage: $0 <output directory> [headline pop_fused pop_two_op long layer5 model]" >&2; exit 2; }
+[ -n "$1" ] || { echo "usage: $0 <output directory> [headline pop_fused pop_two_op long layer5 layer_ops model]" >&2; exit 2; }
 mkdir -p "$1"
 O=$(cd "$1" && pwd)
 shift
-LEGS=${*:-headline pop_fused pop_two_op long layer5 model}
+LEGS=${*:-headline pop_fused pop_two_op long layer5 layer_ops model}
 STEPS=8
 cd /tmp && export TMPDIR=/tmp
 run() { name=$1; shift; echo "[profile] $name" ; timeout -s KILL 150 rocprofv3 "$@" --output-format csv -d "$O/$name" -o r -- $CMD > "$O/$name.log" 2>&1; }

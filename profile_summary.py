@@ -16,7 +16,7 @@ import subprocess
 import sys
 from collections import defaultdict
 
-OURS = ("retention_", "suffix_intra", "segment_scan", "segment_contrib", "decode_step", "rotary_qk", "gated_norm")
+OURS = ("retention_", "suffix_intra", "short_seq", "segment_scan", "segment_contrib", "decode_step", "rotary_qk", "gated_norm")
 COPY_KIB = 1 << 20   # the calibration copies 1 GiB
 
 
@@ -54,7 +54,7 @@ def copy_reading(path, counter):
 
 
 FAMILIES = (
-    ("retention kernels of this library", ("retention_", "suffix_intra", "segment_scan", "segment_contrib", "decode_step")),
+    ("retention kernels of this library", ("retention_", "suffix_intra", "short_seq", "segment_scan", "segment_contrib", "decode_step")),
     ("rotary embedding kernel of this library", ("rotary_qk",)),
     ("norm + gate kernels of this library", ("gated_norm",)),
     ("GEMMs (rocBLAS / hipBLASLt)", ("Cijk_", "gemm", "Gemm")),
@@ -99,6 +99,7 @@ LEGS = (
     ("pop_two_op", "config 4 through the reference's call sequence (flash_pop_retention, torch.cat, fused_chunk_retention)"),
     ("long", "config 3: B2 H8 T16384 dk128 dv256 with carried state (split-sequence entry points)"),
     ("layer5", "the retention op of one layer of config 5: fused POP step, B8 T2048 H12 dk64 dv128"),
+    ("layer_ops", "the elementwise stages around the op at config 2's tensor shapes (B8 T4096 H16 d128): rotary, norm + gate forward and backward"),
 )
 
 
@@ -155,7 +156,7 @@ def main():
             if not os.path.exists(path):
                 continue
             cs = counters(path)
-            names = sorted(k for k in cs if any(o in k for o in ("retention_", "suffix_intra", "segment_contrib")))
+            names = sorted(k for k in cs if any(o in k for o in ("retention_", "suffix_intra", "segment_contrib", "short_seq", "rotary_qk", "gated_norm")))
             ctrs = sorted({c for k in names for c in cs[k]})
             print(f"\n## Shader counters per launch ({run})\n")
             print("| counter | " + " | ".join(names) + " |\n|---|" + "---|" * len(names))

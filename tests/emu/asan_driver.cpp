@@ -31,6 +31,16 @@ int done(int rc, const char* what, int B, int T, int H, int dk, int dv, int extr
   return rc;
 }
 
+// many short sequences with a state each and no gradient of the final state: the suffix call of the POP layer
+int short_sequences(int B, int T, int H, int dk, int dv, bool state) {
+  std::vector<double> dec(H, 0.97);
+  const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
+  uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = state ? buf(ns) : nullptr;
+  uint16_t *dO = buf(nv), *dq = buf(nq, false), *dk_ = buf(nq, false), *dv_ = buf(nv, false), *ds0 = state ? buf(ns, false) : nullptr;
+  const int rc = fp_retention_bwd(q, k, v, s, dec.data(), dO, nullptr, dq, dk_, dv_, ds0, B, T, H, dk, dv, nullptr);
+  return done(rc, "short", B, T, H, dk, dv, state);
+}
+
 int plain(int B, int T, int H, int dk, int dv, bool split) {
   std::vector<double> dec(H, 0.97);
   const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
@@ -152,7 +162,13 @@ int main() {
   rc |= plain(1, 530, 1, 64, 64, false);      // 64 x 64 states (half of the waves own a tile), ragged last chunk,
   rc |= checkpointed(1, 600, 1, 256, 64, 128);   // checkpoints of 64 x 128 states
   rc |= fused(1, 8, 64, 9, 1, 64, 64);        // folded suffixes of 9 tokens on 64 x 64 states
+  rc |= pop(1, 640, 1, 128, 128, 64);         // gradients of block states added on the reverse walk of that kernel
+  rc |= pop(1, 700, 1, 64, 128, 128);         // ... 64-wide keys, tokens after the last boundary
   fp_set_backward_choice(0, -1);
+  rc |= short_sequences(7, 16, 2, 128, 128, true);   // more pairs than workgroups, one k-step along the tokens
+  rc |= short_sequences(2, 31, 1, 64, 128, true);    // two k-steps, 64-wide keys
+  rc |= short_sequences(3, 5, 1, 128, 64, false);    // no state
+  rc |= short_sequences(1, 32, 2, 64, 64, true);
   rc |= decode(2, 3, 64, 128);
   rc |= decode(1, 1, 256, 256);
   rc |= rotary(3, 11, 2, 64, true);           // last workgroup partly idle

@@ -5,6 +5,7 @@
 #include "segment_scan.h"
 #include "segment_contrib.h"
 #include "retention_bwd_fused.h"
+#include "short_seq.h"
 #include "decode_step.h"
 #include "layer_ops.h"
 
@@ -75,6 +76,9 @@ namespace {
 
 template <int DK, int DV>
 int emu_bwd_fused(const fpk::FusedBwdArgs& a) {
+  if (a.d_blocks)
+    return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_BLOCKS),
+                    [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_BLOCKS>(a, l, fprt::block_index()); });
   if (a.fold) {
     if (int rc = run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_FOLD),
                           [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_FOLD>(a, l, fprt::block_index()); }))
@@ -102,6 +106,21 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const 
   if (a.dk_dim == 64 && a.dv_dim == 128) return emu_bwd_fused<64, 128>(a);
   if (a.dk_dim == 128 && a.dv_dim == 64) return emu_bwd_fused<128, 64>(a);
   return emu_bwd_fused<64, 64>(a);
+}
+
+int fpk_launch_short_bwd(const fpk::FusedBwdArgs& a, void* /*stream*/, const char** err) {
+  if (const char* why = fpk::check_short_seq_bwd(a)) {
+    *err = why;
+    return 1;
+  }
+  const int pairs = a.B * a.H, nwg = pairs < 3 ? pairs : 3;   // several pairs per workgroup
+  if (a.dk_dim == 128 && a.dv_dim == 128)
+    return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(128, 128), [&](char* l) { fpk::short_seq_bwd<128, 128>(a, l); });
+  if (a.dk_dim == 64 && a.dv_dim == 128)
+    return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(64, 128), [&](char* l) { fpk::short_seq_bwd<64, 128>(a, l); });
+  if (a.dk_dim == 128 && a.dv_dim == 64)
+    return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(128, 64), [&](char* l) { fpk::short_seq_bwd<128, 64>(a, l); });
+  return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(64, 64), [&](char* l) { fpk::short_seq_bwd<64, 64>(a, l); });
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* /*stream*/, const char** err) {

@@ -82,6 +82,31 @@ def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
                 ("ds0", ds0, gs)])
 
 
+@pytest.mark.parametrize("B,T,H,dk,dv,block,state_std", [
+    (1, 640, 1, 128, 128, 64, 0.5),     # a block state behind every chunk, the last one at the end of the sequence
+    (1, 700, 2, 64, 128, 128, 0.5),     # two chunks per block, tokens after the last block boundary
+    (1, 768, 1, 128, 64, 256, None),    # the sequence ends on a block boundary, no initial state
+    (1, 600, 1, 64, 64, 192, 0.3),      # 64 x 64 states
+    (1, 520, 1, 128, 128, 576, 0.5),    # no full block: nothing to add
+])
+def test_pop_backward_in_the_kernel_that_carries_ds_once(emu_lib, choose_backward, B, T, H, dk, dv, block, state_std):
+    """flash_pop_retention's backward with whole chunks per block: the gradients of the block states join dS in the
+    fused backward where its reverse walk crosses their boundaries.  Against the oracle and the pass-per-gradient path."""
+    decays = oracle.head_decays(H, (5, 12))
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + block, state_std=state_std)
+    d_o, d_b = hp.make_cotangents([(B, T, H, dv), (B, T // block, H, dk, dv)], seed=T)
+    choose_backward(FUSED)
+    grads = hp.raw_pop_bwd(emu_lib, q, k, v, s, decays, block, d_o, d_b)
+    _, _, ref = hp.oracle_pop(q, k, v, s, decays, block, d_o, d_b)
+    _check_all([(n, g, r) for n, g, r in zip(("dq", "dk", "dv", "ds0"), grads, ref)])
+    choose_backward(PASSES)
+    other = hp.raw_pop_bwd(emu_lib, q, k, v, s, decays, block, d_o, d_b)
+    assert not all(torch.equal(x, y) for x, y in zip(grads, other) if x is not None), "both calls took the same kernels"
+    for n, x, y in zip(("dq", "dk", "dv", "ds0"), grads, other):
+        if x is not None:
+            assert hp.error_report(x, y.float())["rms_ratio"] < 0.004, n
+
+
 FUSED_NAMES = ("dq", "dk", "dv", "dq_sfx", "dk_sfx", "dv_sfx", "ds0")
 
 
@@ -207,6 +232,37 @@ def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, stat
     choose_backward(PASSES)
     g3 = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, d_s)
     assert not torch.equal(g3[1], dk_)
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,state_std,want_ds0", [
+    (5, 16, 2, 128, 128, 0.5, True),     # more (sequence, head) pairs than the harness runs workgroups
+    (7, 31, 1, 64, 128, 0.5, True),      # two k-steps along the tokens, 64-wide keys
+    (3, 9, 2, 128, 64, None, True),      # no state: no read-out, no d_s0
+    (4, 32, 1, 64, 64, 0.3, True),       # the longest sequence the kernel takes
+    (2, 1, 3, 128, 128, 0.5, True),      # one token
+    (3, 17, 2, 64, 128, 0.5, False),     # d_s0 not wanted
+])
+def test_backward_for_many_short_sequences(emu_lib, choose_backward, B, T, H, dk, dv, state_std, want_ds0):
+    """At most 32 tokens per sequence, a state per sequence, no gradient of the final state (the suffix call of
+    the reference's POP layer): the backward takes one (sequence, head) pair per step in a kernel of its own."""
+    decays = oracle.head_decays(H, (4, 9))
+    q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + dk, state_std=state_std)
+    d_o, = hp.make_cotangents([(B, T, H, dv)], seed=T + 1)
+    grads = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None, want_ds0=want_ds0)
+    _, _, ref = hp.oracle_plain(q, k, v, s, decays, d_o, None)
+    _check_all([(n, g, r) for n, g, r in zip(("dq", "dk", "dv", "ds0"), grads, ref) if g is not None])
+    choose_backward(PASSES)
+    other = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None, want_ds0=want_ds0)
+    for n, x, y in zip(("dq", "dk", "dv", "ds0"), grads, other):
+        if x is not None:
+            assert hp.error_report(x, y.float())["rms_ratio"] < 0.004, n
+    # with a gradient of the final state the chunk kernels run, and give the same dq (the short kernel's only
+    # state term) up to the rounding of its partial sums
+    d_s, = hp.make_cotangents([(B, H, dk, dv)], seed=T + 2)
+    choose_backward(0)
+    with_ds = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, d_s, want_ds0=want_ds0)
+    _, _, ref_ds = hp.oracle_plain(q, k, v, s, decays, d_o, d_s)
+    _check_all([(n, g, r) for n, g, r in zip(("dq", "dk", "dv", "ds0"), with_ds, ref_ds) if g is not None])
 
 
 def test_c_entry_points_refuse_a_capturing_stream(emu_lib):

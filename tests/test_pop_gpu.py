@@ -48,9 +48,22 @@ def run_pop(B, T, H, dk, dv, block, state_std, seed, decay_range=(5, 12), oracle
     (1, 40, 2, 64, 64, 100),       # no full block: empty block_states
     (1, 192, 2, 128, 256, 64),
     (2, 300, 2, 192, 64, 48),      # 192-wide keys: three visits per chunk, block states written and their gradients read
+    (8, 1024, 12, 64, 128, 64),    # 96 streams, whole chunks per block: the backward that carries dS once adds the block-state gradients on its way
+    (6, 832, 16, 128, 128, 128),   # ... two chunks per block, tokens after the last boundary
+    (11, 768, 8, 128, 64, 256),    # ... the sequence ends on a block boundary
 ])
 def test_pop_parity_sweep(B, T, H, dk, dv, block):
     run_pop(B, T, H, dk, dv, block, 0.3, seed=T + block)
+
+
+@pytest.mark.parametrize("choice", [1, 2])
+def test_pop_backward_forced_choice(hip_lib, choice):
+    """Both backward paths of a shape with whole chunks per block (8 streams: the passes by shape), against the oracle."""
+    assert hip_lib.fp_set_backward_choice(choice, -1) == 0
+    try:
+        run_pop(2, 640, 4, 64, 128, 128, 0.3, seed=choice)
+    finally:
+        assert hip_lib.fp_set_backward_choice(0, -1) == 0
 
 
 def test_pop_without_state_argument():

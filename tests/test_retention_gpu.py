@@ -29,7 +29,10 @@ def run_plain(B, T, H, dk, dv, state_std, seed, decay_range=None, with_ds=True, 
     leaves = [None if t is None else t.to(DEV).requires_grad_() for t in (q, k, v, s)]
     o, S = fused_chunk_retention(*leaves, decays)
     assert o.dtype == torch.bfloat16 and o.is_contiguous() and S.shape == (B, H, dk, dv)
-    torch.autograd.backward([o, S], [d_o.to(DEV), d_s.to(DEV) if with_ds else torch.zeros_like(S)])
+    if with_ds is None:   # nobody differentiates the final state
+        torch.autograd.backward([o], [d_o.to(DEV)])
+    else:
+        torch.autograd.backward([o, S], [d_o.to(DEV), d_s.to(DEV) if with_ds else torch.zeros_like(S)])
     torch.cuda.synchronize()
     bsel = list(range(B)) if oracle_batches is None else oracle_batches
     for b in bsel:
@@ -86,6 +89,21 @@ def test_forced_backward_choice(hip_lib, choice, B, T, H, dk, dv):
         run_plain(B, T, H, dk, dv, 0.1, seed=T + choice)
     finally:
         assert hip_lib.fp_set_backward_choice(0, -1) == 0
+
+
+@pytest.mark.parametrize("B,T,H,dk,dv,state_std", [
+    (520, 16, 16, 128, 128, 0.3),    # the suffix batch of benchmark configuration 4: 8 320 (sequence, head) pairs
+    (264, 16, 12, 64, 128, 0.3),     # ... of configuration 5
+    (40, 31, 4, 128, 64, 0.3),       # the suffix length of the reference's model tests (tests/test_pop_retnet.py:35)
+    (3, 32, 2, 64, 64, None),        # fewer pairs than compute units, no state
+    (9, 1, 5, 128, 128, 0.5),        # single tokens
+])
+def test_many_short_sequences_without_final_state_gradient(B, T, H, dk, dv, state_std):
+    """At most 32 tokens per sequence and nothing differentiating the final states: the backward of the suffix call
+    of the reference's POP layer (flash_pop/pop_retnet.py:163-168 discards the final states), one (sequence, head)
+    pair per step in a kernel of its own.  Oracle on the GPU, a spread of sequences."""
+    step = max(1, B // 7)
+    run_plain(B, T, H, dk, dv, state_std, seed=T + B, with_ds=None, oracle_batches=list(range(0, B, step)), oracle_device=DEV)
 
 
 def test_decay_range_of_reference_tests():
