@@ -230,13 +230,18 @@ bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes 
   const int choice = g_bwd_choice.load(std::memory_order_relaxed);
   if (choice == BWD_PASSES) return false;
   if (choice == BWD_FUSED) return true;
-  // two workgroups per stream: with fewer than two thirds of the compute units covered the column-tiled
-  // passes, which fill the chip, are faster (256 units, T = 4096: 64 streams 0.33 ms against 0.30 ms).  With POP
-  // suffixes the passes pay for every suffix as a stop of each of their four walks and this kernel does not:
-  // it wins from 3/16 of the units' worth of streams on (48 streams, 64-token blocks: 0.44 against 0.57 ms; 512-token
-  // blocks: even between 48 and 80 streams; 32 streams: the passes by 8 %)
-  if (pop_suffixes) return 16LL * s.B * s.H >= 3LL * fpk_compute_units();
-  return 3LL * s.B * s.H >= fpk_compute_units();
+  // Two workgroups per stream against column-tiled passes that fill the chip: the fused kernel needs enough streams.
+  // Measured cross-overs on a 256-unit device (forward + backward at T = 2048 .. 4096; streams = B * H):
+  //                 dk = dv = 128      dk 64, dv 128      dk 128, dv 64      dk = dv = 64
+  //   plain         86  (3 s >= CU)    32  (8 s >= CU)    64  (4 s >= CU)    64  (4 s >= CU)
+  //   POP suffixes  48  (16 s >= 3 CU) 32  (8 s >= CU)    32  (8 s >= CU)    96  (8 s >= 3 CU)
+  // (d = 128, 64 streams: 0.33 ms fused against 0.30 ms in passes at T = 4096; with suffixes the passes pay for every
+  // suffix as a stop of each of their four walks and this kernel does not: 48 streams, 64-token blocks, 0.44 against
+  // 0.57 ms.  Narrower states make the fused kernel's chunk step cheaper sooner than they help the passes.)
+  const long long streams = (long long)s.B * s.H, cu = fpk_compute_units();
+  const bool wide = s.dk == fpk::FB_D && s.dv == fpk::FB_D, narrow = s.dk == 64 && s.dv == 64;
+  if (pop_suffixes) return wide ? 16 * streams >= 3 * cu : narrow ? 8 * streams >= 3 * cu : 8 * streams >= cu;
+  return wide ? 3 * streams >= cu : s.dk == 64 && s.dv == fpk::FB_D ? 8 * streams >= cu : 4 * streams >= cu;
 }
 
 // Tokens between the states that fp_retention_fwd_ckpt leaves for the backward (0: none wanted).
