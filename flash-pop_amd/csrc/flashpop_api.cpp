@@ -225,11 +225,11 @@ bool fused_dim(int d) { return d == 64 || d == 128; }
 bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes = false, int block = 0) {
   if (!fused_dim(s.dk) || !fused_dim(s.dv)) return false;
   if (d_blocks && (block <= 0 || block % fpk::CH != 0)) return false;
-  if (s.T < 8 * fpk::CH) return false;   // short sequences: the walk over many of them per workgroup serves better
   read_environment();
   const int choice = g_bwd_choice.load(std::memory_order_relaxed);
   if (choice == BWD_PASSES) return false;
-  if (choice == BWD_FUSED) return true;
+  if (choice == BWD_FUSED) return true;   // whatever the length and the number of streams
+  if (s.T < 8 * fpk::CH) return false;    // short sequences: the walk over many of them per workgroup serves better
   // Two workgroups per stream against column-tiled passes that fill the chip: the fused kernel needs enough streams.
   // Measured cross-overs on a 256-unit device (forward + backward at T = 2048 .. 4096; streams = B * H):
   //                 dk = dv = 128      dk 64, dv 128      dk 128, dv 64      dk = dv = 64

@@ -153,17 +153,17 @@ int main() {
   rc |= fused(1, 1, 80, 5, 1, 64, 128, 30);   // tokens after the last block boundary
   rc |= fused(1, 0, 90, 12, 1, 64, 64, 70);   // no full block
   rc |= fused(1, 2, 64, 100, 1, 128, 64);     // suffixes in two parts
-  fp_set_backward_choice(2, -1);        // one stream would not take this path by itself
-  rc |= fused(1, 8, 64, 16, 1, 128, 128);     // backward in the kernel that carries dS once, suffixes as extra stops
-  rc |= plain(1, 530, 1, 128, 128, false);    // the same kernel without suffixes, ragged last chunk
-  rc |= checkpointed(1, 600, 1, 128);         // ... with the forward's checkpoints
-  rc |= fused(1, 8, 64, 16, 1, 64, 128);      // the same kernels for 64-wide keys: folded suffixes,
-  rc |= fused(1, 4, 128, 40, 1, 128, 64);     // 64-wide values with the suffixes as stops,
-  rc |= plain(1, 530, 1, 64, 64, false);      // 64 x 64 states (half of the waves own a tile), ragged last chunk,
-  rc |= checkpointed(1, 600, 1, 256, 64, 128);   // checkpoints of 64 x 128 states
-  rc |= fused(1, 8, 64, 9, 1, 64, 64);        // folded suffixes of 9 tokens on 64 x 64 states
-  rc |= pop(1, 640, 1, 128, 128, 64);         // gradients of block states added on the reverse walk of that kernel
-  rc |= pop(1, 700, 1, 64, 128, 128);         // ... 64-wide keys, tokens after the last boundary
+  fp_set_backward_choice(2, -1);        // one short stream would not take this path by itself
+  rc |= fused(1, 4, 64, 16, 1, 128, 128);     // backward in the kernel that carries dS once, suffixes as extra stops
+  rc |= plain(1, 210, 1, 128, 128, false);    // the same kernel without suffixes, ragged last chunk
+  rc |= checkpointed(1, 280, 1, 128);         // ... with the forward's checkpoints
+  rc |= fused(1, 4, 64, 16, 1, 64, 128);      // the same kernels for 64-wide keys: folded suffixes,
+  rc |= fused(1, 2, 128, 40, 1, 128, 64);     // 64-wide values with the suffixes as stops,
+  rc |= plain(1, 210, 1, 64, 64, false);      // 64 x 64 states (half of the waves own a tile), ragged last chunk,
+  rc |= checkpointed(1, 280, 1, 64, 64, 128);    // checkpoints of 64 x 128 states
+  rc |= fused(1, 4, 64, 9, 1, 64, 64);        // folded suffixes of 9 tokens on 64 x 64 states
+  rc |= pop(1, 256, 1, 128, 128, 64);         // gradients of block states added on the reverse walk of that kernel
+  rc |= pop(1, 300, 1, 64, 128, 128);         // ... 64-wide keys, tokens after the last boundary
   fp_set_backward_choice(0, -1);
   rc |= short_sequences(7, 16, 2, 128, 128, true);   // more pairs than workgroups, one k-step along the tokens
   rc |= short_sequences(2, 31, 1, 64, 128, true);    // two k-steps, 64-wide keys

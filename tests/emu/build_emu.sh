@@ -14,6 +14,11 @@ pids=""
 for w in 64 128 192 256; do
   "$cxx" $flags -DEMU_FAMILY=$w -c "$here/pass_family.cpp" -o "$obj/pass_$w.o" & pids="$pids $!"
 done
+for dk in 64 128; do
+  for dv in 64 128; do
+    "$cxx" $flags -DEMU_DK=$dk -DEMU_DV=$dv -c "$here/fused_family.cpp" -o "$obj/fused_${dk}_$dv.o" & pids="$pids $!"
+  done
+done
 "$cxx" $flags -c "$here/launch_emu.cpp" -o "$obj/launch_emu.o" & pids="$pids $!"
 "$cxx" $flags -c "$csrc/flashpop_api.cpp" -o "$obj/flashpop_api.o" & pids="$pids $!"
 if [ -n "$EMU_MAIN" ]; then

@@ -72,28 +72,15 @@ int fpk_stream_is_capturing(void* /*stream*/) { return g_emu_capturing; }
 // ones take on a real device (several sequences per workgroup, split sequences).
 int fpk_compute_units() { return 8; }
 
-namespace {
-
-template <int DK, int DV>
-int emu_bwd_fused(const fpk::FusedBwdArgs& a) {
-  if (a.d_blocks)
-    return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_BLOCKS),
-                    [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_BLOCKS>(a, l, fprt::block_index()); });
-  if (a.fold) {
-    if (int rc = run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_FOLD),
-                          [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_FOLD>(a, l, fprt::block_index()); }))
-      return rc;
-    const int pairs = a.B * (a.T / a.block + 1) * a.H;
-    return run_grid(fpk::SI_THREADS, pairs < 3 ? pairs : 3, fpk::si_lds_bytes(DK, DV), [&](char* l) { fpk::suffix_intra_bwd<DK, DV>(a, l); });
-  }
-  if (a.block > 0)
-    return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_STOPS),
-                    [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_STOPS>(a, l, fprt::block_index()); });
-  return run_grid(fpk::FB_THREADS, 2 * a.B * a.H, fpk::fb_lds_bytes(DK, DV, fpk::FB_PLAIN),
-                  [&](char* l) { fpk::fused_bwd<DK, DV, fpk::FB_PLAIN>(a, l, fprt::block_index()); });
-}
-
-}  // namespace
+// one translation unit per pair of head dimensions (fused_family.cpp)
+#define EMU_FUSED_FAMILY(DK, DV)                                  \
+  int emu_bwd_fused_##DK##_##DV(const fpk::FusedBwdArgs& a);      \
+  int emu_short_bwd_##DK##_##DV(const fpk::FusedBwdArgs& a);
+EMU_FUSED_FAMILY(128, 128)
+EMU_FUSED_FAMILY(64, 128)
+EMU_FUSED_FAMILY(128, 64)
+EMU_FUSED_FAMILY(64, 64)
+#undef EMU_FUSED_FAMILY
 
 int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const char** err) {
   fpk::FusedBwdArgs a = args;
@@ -102,10 +89,10 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const 
     *err = why;
     return 1;
   }
-  if (a.dk_dim == 128 && a.dv_dim == 128) return emu_bwd_fused<128, 128>(a);
-  if (a.dk_dim == 64 && a.dv_dim == 128) return emu_bwd_fused<64, 128>(a);
-  if (a.dk_dim == 128 && a.dv_dim == 64) return emu_bwd_fused<128, 64>(a);
-  return emu_bwd_fused<64, 64>(a);
+  if (a.dk_dim == 128 && a.dv_dim == 128) return emu_bwd_fused_128_128(a);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return emu_bwd_fused_64_128(a);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return emu_bwd_fused_128_64(a);
+  return emu_bwd_fused_64_64(a);
 }
 
 int fpk_launch_short_bwd(const fpk::FusedBwdArgs& a, void* /*stream*/, const char** err) {
@@ -113,14 +100,10 @@ int fpk_launch_short_bwd(const fpk::FusedBwdArgs& a, void* /*stream*/, const cha
     *err = why;
     return 1;
   }
-  const int pairs = a.B * a.H, nwg = pairs < 3 ? pairs : 3;   // several pairs per workgroup
-  if (a.dk_dim == 128 && a.dv_dim == 128)
-    return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(128, 128), [&](char* l) { fpk::short_seq_bwd<128, 128>(a, l); });
-  if (a.dk_dim == 64 && a.dv_dim == 128)
-    return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(64, 128), [&](char* l) { fpk::short_seq_bwd<64, 128>(a, l); });
-  if (a.dk_dim == 128 && a.dv_dim == 64)
-    return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(128, 64), [&](char* l) { fpk::short_seq_bwd<128, 64>(a, l); });
-  return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(64, 64), [&](char* l) { fpk::short_seq_bwd<64, 64>(a, l); });
+  if (a.dk_dim == 128 && a.dv_dim == 128) return emu_short_bwd_128_128(a);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return emu_short_bwd_64_128(a);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return emu_short_bwd_128_64(a);
+  return emu_short_bwd_64_64(a);
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* /*stream*/, const char** err) {

@@ -83,11 +83,11 @@ def test_pop_fwd_bwd(emu_lib, B, T, H, dk, dv, block):
 
 
 @pytest.mark.parametrize("B,T,H,dk,dv,block,state_std", [
-    (1, 640, 1, 128, 128, 64, 0.5),     # a block state behind every chunk, the last one at the end of the sequence
-    (1, 700, 2, 64, 128, 128, 0.5),     # two chunks per block, tokens after the last block boundary
-    (1, 768, 1, 128, 64, 256, None),    # the sequence ends on a block boundary, no initial state
-    (1, 600, 1, 64, 64, 192, 0.3),      # 64 x 64 states
-    (1, 520, 1, 128, 128, 576, 0.5),    # no full block: nothing to add
+    (1, 256, 1, 128, 128, 64, 0.5),     # a block state behind every chunk, the last one at the end of the sequence
+    (1, 330, 2, 64, 128, 128, 0.5),     # two chunks per block, tokens after the last block boundary
+    (1, 256, 1, 128, 64, 128, None),    # the sequence ends on a block boundary, no initial state
+    (1, 300, 1, 64, 64, 192, 0.3),      # 64 x 64 states
+    (1, 200, 1, 128, 128, 576, 0.5),    # no full block: nothing to add
 ])
 def test_pop_backward_in_the_kernel_that_carries_ds_once(emu_lib, choose_backward, B, T, H, dk, dv, block, state_std):
     """flash_pop_retention's backward with whole chunks per block: the gradients of the block states join dS in the
@@ -165,16 +165,17 @@ def test_split_sequences_fwd_bwd(emu_lib, B, T, H, dk, dv, state_std, segments):
 
 
 @pytest.mark.parametrize("B,nblk,block,Ls,H,state_std,dk,dv", [
-    (1, 4, 128, 16, 1, 0.5, 128, 128),     # two chunks per block
-    (1, 8, 64, 64, 1, None, 128, 128),     # block == chunk, suffixes as long as a chunk, no initial state
-    (1, 3, 192, 1, 2, 0.3, 128, 128),      # three chunks per block, one-token suffixes, two heads
+    (1, 2, 128, 16, 1, 0.5, 128, 128),     # two chunks per block
+    (1, 4, 64, 64, 1, None, 128, 128),     # block == chunk, suffixes as long as a chunk, no initial state
+    (1, 1, 192, 1, 2, 0.3, 128, 128),      # three chunks per block, one-token suffixes, two heads
     (1, 8, 64, 9, 1, 0.3, 128, 128),       # short suffixes folded into every chunk; 9 suffixes over 3 workgroups of the second kernel
-    (1, 8, 64, 16, 2, 0.3, 64, 128),       # 64-wide keys: folded suffixes
-    (1, 4, 128, 40, 1, None, 128, 64),     # 64-wide values: suffixes as stops, no initial state
-    (1, 8, 64, 9, 1, 0.5, 64, 64),         # 64 x 64 states: four state tiles for eight waves
+    (1, 4, 64, 16, 2, 0.3, 64, 128),       # 64-wide keys: folded suffixes
+    (1, 2, 128, 40, 1, None, 128, 64),     # 64-wide values: suffixes as stops, no initial state
+    (1, 4, 64, 9, 1, 0.5, 64, 64),         # 64 x 64 states: four state tiles for eight waves
 ])
 def test_fused_pop_backward_that_carries_ds_once(emu_lib, choose_backward, B, nblk, block, Ls, H, state_std, dk, dv):
-    """dk, dv of 64 or 128, whole chunks per block, at least eight chunks: the fused POP backward runs in
+    """dk, dv of 64 or 128, whole chunks per block (forced here at lengths below the eight chunks from which the
+    library chooses it by itself): the fused POP backward runs in
     the kernel that walks backward once for dk and dv beside a forward walk for dq, with the
     suffixes as extra stops at the block boundaries or folded into the chunks there.  Same results as the
     pass-per-gradient path."""
@@ -198,17 +199,18 @@ def test_fused_pop_backward_that_carries_ds_once(emu_lib, choose_backward, B, nb
 
 
 @pytest.mark.parametrize("B,T,H,state_std,every,dk,dv", [
-    (1, 700, 1, 0.5, 128, 128, 128),      # ragged tail beyond the last checkpoint, initial state
-    (1, 512, 1, None, 256, 128, 128),     # the sequence ends on a checkpoint, no initial state
-    (2, 520, 1, 0.3, 64, 128, 128),       # a checkpoint after every chunk, two sequences
-    (1, 600, 1, 0.2, 1024, 128, 128),     # interval longer than the sequence: no checkpoint at all
-    (1, 576, 1, 0.4, 0, 128, 128),        # no checkpoint buffer: the fused backward walks forward from s0
-    (1, 700, 2, 0.5, 256, 64, 128),       # 64-wide keys
-    (1, 530, 1, None, 0, 128, 64),        # 64-wide values, no checkpoints, no initial state
-    (1, 600, 1, 0.3, 128, 64, 64),        # 64 x 64 states
+    (1, 330, 1, 0.5, 128, 128, 128),      # ragged tail beyond the last checkpoint, initial state
+    (1, 256, 1, None, 128, 128, 128),     # the sequence ends on a checkpoint, no initial state
+    (2, 200, 1, 0.3, 64, 128, 128),       # a checkpoint after every chunk, two sequences
+    (1, 200, 1, 0.2, 1024, 128, 128),     # interval longer than the sequence: no checkpoint at all
+    (1, 260, 1, 0.4, 0, 128, 128),        # no checkpoint buffer: the fused backward walks forward from s0
+    (1, 330, 2, 0.5, 128, 64, 128),       # 64-wide keys
+    (1, 210, 1, None, 0, 128, 64),        # 64-wide values, no checkpoints, no initial state
+    (1, 300, 1, 0.3, 128, 64, 64),        # 64 x 64 states
 ])
 def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, state_std, every, dk, dv):
-    """dk, dv of 64 or 128 and at least eight chunks: the backward that carries dS once, beside the
+    """dk, dv of 64 or 128 (forced here at lengths below the eight chunks from which the library chooses it by
+    itself): the backward that carries dS once, beside the
     workgroup that re-runs the state from the checkpoints the forward left (segments taken from
     the last to the first)."""
     choose_backward(FUSED)
