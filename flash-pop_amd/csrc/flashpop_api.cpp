@@ -200,8 +200,34 @@ void transposed_state(fpk::PassArgs& a, const Shape& s) {
   a.rs_n = s.dv;
 }
 
+// Sequences of at most fpk::SS_ROWS tokens with head dimensions of 64 or 128: the forward that takes a (sequence,
+// head) pair per step (short_seq.h) instead of a 64-token item per pair and column tile.  Shares the switch of the
+// backward (the pass kernel stays reachable for comparisons).
+bool fused_dim(int d);
+bool use_short_forward(const Shape& s) {
+  if (s.T > fpk::SS_ROWS || !fused_dim(s.dk) || !fused_dim(s.dv)) return false;
+  read_environment();
+  return g_bwd_choice.load(std::memory_order_relaxed) != BWD_PASSES;
+}
+
+int forward_short(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays, void* o,
+                  void* s_out, void* stream) {
+  fpk::ShortFwdArgs a;
+  std::memset(&a, 0, sizeof a);
+  a.q = in(q); a.k = in(k); a.v = in(v); a.s0 = in(s0);
+  a.o = out(o); a.s_out = out(s_out);
+  a.B = s.B; a.T = s.T; a.H = s.H;
+  a.dk_dim = s.dk; a.dv_dim = s.dv;
+  a.scale = 1.0f / std::sqrt((float)s.dk);
+  for (int h = 0; h < s.H; ++h) a.log2g[h] = (float)std::log2(decays[h]);
+  const char* msg = "";
+  if (fpk_launch_short_fwd(a, stream, &msg) != 0) return fail(FP_ERR_LAUNCH, "short-sequence forward: %s", msg);
+  return FP_OK;
+}
+
 int forward(const Shape& s, const void* q, const void* k, const void* v, const void* s0, const double* decays, void* o,
             void* s_out, void* block_states, int block, void* stream) {
+  if (!block_states && block == 0 && use_short_forward(s)) return forward_short(s, q, k, v, s0, decays, o, s_out, stream);
   fpk::PassArgs a;
   fill_common(a, s, decays);
   const float sc = 1.0f / std::sqrt((float)s.dk);

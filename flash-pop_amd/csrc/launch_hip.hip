@@ -52,6 +52,12 @@ __global__ __launch_bounds__(fpk::FB_THREADS) void short_seq_bwd_kernel(const fp
   fpk::short_seq_bwd<DK, DV>(args, lds);
 }
 
+template <int DK, int DV>
+__global__ __launch_bounds__(fpk::FB_THREADS) void short_seq_fwd_kernel(const fpk::ShortFwdArgs args) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  fpk::short_seq_fwd<DK, DV>(args, lds);
+}
+
 __global__ __launch_bounds__(fpk::SCAN_THREADS) void segment_scan_kernel(const fpk::ScanArgs args) {
   fpk::segment_scan(args);
 }
@@ -321,7 +327,28 @@ int launch_short_bwd(const fpk::FusedBwdArgs& a, int slot, hipStream_t st, const
   return launched(err);
 }
 
+template <int DK, int DV>
+int launch_short_fwd(const fpk::ShortFwdArgs& a, int slot, hipStream_t st, const char** err) {
+  constexpr int lds = fpk::ss_fwd_lds_bytes(DK, DV);
+  if (arm(reinterpret_cast<const void*>(short_seq_fwd_kernel<DK, DV>), lds, 64 + 24 + slot, err)) return 1;
+  const long long pairs = (long long)a.B * a.H, wgs = fpk_compute_units();   // one workgroup per unit, as in the backward
+  hipLaunchKernelGGL((short_seq_fwd_kernel<DK, DV>), dim3((unsigned)(pairs < wgs ? pairs : wgs)), dim3(fpk::FB_THREADS), lds, st, a);
+  return launched(err);
+}
+
 }  // namespace
+
+int fpk_launch_short_fwd(const fpk::ShortFwdArgs& a, void* stream, const char** err) {
+  if (const char* why = fpk::check_short_seq_fwd(a)) {
+    *err = why;
+    return 1;
+  }
+  const hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a.dk_dim == 128 && a.dv_dim == 128) return launch_short_fwd<128, 128>(a, 0, st, err);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return launch_short_fwd<64, 128>(a, 1, st, err);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return launch_short_fwd<128, 64>(a, 2, st, err);
+  return launch_short_fwd<64, 64>(a, 3, st, err);
+}
 
 int fpk_launch_short_bwd(const fpk::FusedBwdArgs& a, void* stream, const char** err) {
   if (const char* why = fpk::check_short_seq_bwd(a)) {

@@ -153,6 +153,17 @@ struct FusedBwdArgs {
   float scale;                             // dk^-1/2
   float log2g[MAX_HEADS];
 };
+// Forward for many short sequences (short_seq.h): T <= SS_ROWS.
+struct ShortFwdArgs {
+  const uint16_t *q, *k, *v;               // q, k [B,T,H,dk_dim]; v [B,T,H,dv_dim]
+  const uint16_t* s0;                      // [B,H,dk_dim,dv_dim], nullable (zeros)
+  uint16_t* o;                             // [B,T,H,dv_dim]
+  uint16_t* s_out;                         // [B,H,dk_dim,dv_dim], nullable (not wanted)
+  int B, T, H;
+  int dk_dim, dv_dim;                      // head dimensions: 64 or 128 each
+  float scale;                             // dk^-1/2
+  float log2g[MAX_HEADS];
+};
 constexpr int DECODE_THREADS = 256;
 constexpr int decode_lds_bytes(int dv) { return (DECODE_THREADS / (dv / 8)) * dv * 4; }
 
@@ -212,6 +223,7 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char
 
 // Launches the backward for many short sequences (short_seq.h: T <= 32, no gradient of the final state).
 int fpk_launch_short_bwd(const fpk::FusedBwdArgs& args, void* stream, const char** err);
+int fpk_launch_short_fwd(const fpk::ShortFwdArgs& args, void* stream, const char** err);
 
 // Launches the segment scan.  Same conventions as fpk_launch_pass.
 int fpk_launch_scan(const fpk::ScanArgs& args, void* stream, const char** err);

@@ -37,7 +37,9 @@ int short_sequences(int B, int T, int H, int dk, int dv, bool state) {
   const size_t nq = (size_t)B * T * H * dk, nv = (size_t)B * T * H * dv, ns = (size_t)B * H * dk * dv;
   uint16_t *q = buf(nq), *k = buf(nq), *v = buf(nv), *s = state ? buf(ns) : nullptr;
   uint16_t *dO = buf(nv), *dq = buf(nq, false), *dk_ = buf(nq, false), *dv_ = buf(nv, false), *ds0 = state ? buf(ns, false) : nullptr;
-  const int rc = fp_retention_bwd(q, k, v, s, dec.data(), dO, nullptr, dq, dk_, dv_, ds0, B, T, H, dk, dv, nullptr);
+  uint16_t *o = buf(nv, false), *so = state ? buf(ns, false) : nullptr;   // the final state only for the pairs that have an initial one
+  int rc = fp_retention_fwd(q, k, v, s, dec.data(), o, so, B, T, H, dk, dv, nullptr);
+  if (!rc) rc = fp_retention_bwd(q, k, v, s, dec.data(), dO, nullptr, dq, dk_, dv_, ds0, B, T, H, dk, dv, nullptr);
   return done(rc, "short", B, T, H, dk, dv, state);
 }
 
@@ -57,6 +59,11 @@ int plain(int B, int T, int H, int dk, int dv, bool split) {
     return done(rc, "split", B, T, H, dk, dv, (int)wb);
   }
   rc = fp_retention_fwd(q, k, v, s, dec.data(), o, so, B, T, H, dk, dv, nullptr);
+  if (!rc && T <= 32) {   // short sequences have a forward kernel of their own: the pass kernel's turn
+    fp_set_backward_choice(1, -1);
+    rc = fp_retention_fwd(q, k, v, s, dec.data(), o, so, B, T, H, dk, dv, nullptr);
+    fp_set_backward_choice(0, -1);
+  }
   if (!rc) rc = fp_retention_bwd(q, k, v, s, dec.data(), dO, dS, dq, dk_, dv_, ds0, B, T, H, dk, dv, nullptr);
   return done(rc, "plain", B, T, H, dk, dv, 0);
 }

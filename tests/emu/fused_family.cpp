@@ -1,4 +1,4 @@
-// The fused backward, the kernel for the suffixes folded into it and the backward for many short
+// The fused backward, the kernel for the suffixes folded into it and the two kernels for many short
 // sequences on the CPU thread harness, for ONE pair of head dimensions: compiled once per pair with
 // -DEMU_DK=64|128 -DEMU_DV=64|128, so that the harness builds in parallel.  Test infrastructure only.
 #include "device_rt.h"
@@ -40,4 +40,10 @@ int EMU_NAME(emu_bwd_fused_, EMU_DK, EMU_DV)(const fpk::FusedBwdArgs& a) {
 int EMU_NAME(emu_short_bwd_, EMU_DK, EMU_DV)(const fpk::FusedBwdArgs& a) {
   const int pairs = a.B * a.H, nwg = pairs < 3 ? pairs : 3;   // several pairs per workgroup
   return run_grid(fpk::FB_THREADS, nwg, fpk::ss_lds_bytes(DK, DV), [&](char* l) { fpk::short_seq_bwd<DK, DV>(a, l); });
+}
+
+// `a` has passed check_short_seq_fwd
+int EMU_NAME(emu_short_fwd_, EMU_DK, EMU_DV)(const fpk::ShortFwdArgs& a) {
+  const int pairs = a.B * a.H, nwg = pairs < 3 ? pairs : 3;
+  return run_grid(fpk::FB_THREADS, nwg, fpk::ss_fwd_lds_bytes(DK, DV), [&](char* l) { fpk::short_seq_fwd<DK, DV>(a, l); });
 }

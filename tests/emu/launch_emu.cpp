@@ -75,7 +75,8 @@ int fpk_compute_units() { return 8; }
 // one translation unit per pair of head dimensions (fused_family.cpp)
 #define EMU_FUSED_FAMILY(DK, DV)                                  \
   int emu_bwd_fused_##DK##_##DV(const fpk::FusedBwdArgs& a);      \
-  int emu_short_bwd_##DK##_##DV(const fpk::FusedBwdArgs& a);
+  int emu_short_bwd_##DK##_##DV(const fpk::FusedBwdArgs& a);      \
+  int emu_short_fwd_##DK##_##DV(const fpk::ShortFwdArgs& a);
 EMU_FUSED_FAMILY(128, 128)
 EMU_FUSED_FAMILY(64, 128)
 EMU_FUSED_FAMILY(128, 64)
@@ -104,6 +105,17 @@ int fpk_launch_short_bwd(const fpk::FusedBwdArgs& a, void* /*stream*/, const cha
   if (a.dk_dim == 64 && a.dv_dim == 128) return emu_short_bwd_64_128(a);
   if (a.dk_dim == 128 && a.dv_dim == 64) return emu_short_bwd_128_64(a);
   return emu_short_bwd_64_64(a);
+}
+
+int fpk_launch_short_fwd(const fpk::ShortFwdArgs& a, void* /*stream*/, const char** err) {
+  if (const char* why = fpk::check_short_seq_fwd(a)) {
+    *err = why;
+    return 1;
+  }
+  if (a.dk_dim == 128 && a.dv_dim == 128) return emu_short_fwd_128_128(a);
+  if (a.dk_dim == 64 && a.dv_dim == 128) return emu_short_fwd_64_128(a);
+  if (a.dk_dim == 128 && a.dv_dim == 64) return emu_short_fwd_128_64(a);
+  return emu_short_fwd_64_64(a);
 }
 
 int fpk_launch_contrib(const fpk::ContribArgs& a, void* /*stream*/, const char** err) {

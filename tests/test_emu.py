@@ -244,16 +244,24 @@ def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, stat
     (2, 1, 3, 128, 128, 0.5, True),      # one token
     (3, 17, 2, 64, 128, 0.5, False),     # d_s0 not wanted
 ])
-def test_backward_for_many_short_sequences(emu_lib, choose_backward, B, T, H, dk, dv, state_std, want_ds0):
-    """At most 32 tokens per sequence, a state per sequence, no gradient of the final state (the suffix call of
-    the reference's POP layer): the backward takes one (sequence, head) pair per step in a kernel of its own."""
+def test_many_short_sequences(emu_lib, choose_backward, B, T, H, dk, dv, state_std, want_ds0):
+    """At most 32 tokens per sequence, a state per sequence (the suffix call of the reference's POP layer): forward
+    and, with no gradient of the final state, backward take one (sequence, head) pair per step in kernels of their
+    own."""
     decays = oracle.head_decays(H, (4, 9))
     q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T + dk, state_std=state_std)
     d_o, = hp.make_cotangents([(B, T, H, dv)], seed=T + 1)
+    o, S = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+    o_only, none = hp.raw_fwd(emu_lib, q, k, v, s, decays, want_state=False)
     grads = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None, want_ds0=want_ds0)
-    _, _, ref = hp.oracle_plain(q, k, v, s, decays, d_o, None)
+    o_ref, S_ref, ref = hp.oracle_plain(q, k, v, s, decays, d_o, None)
+    _check_all([("o", o, o_ref), ("S", S, S_ref)])
+    assert none is None and torch.equal(o_only, o)
     _check_all([(n, g, r) for n, g, r in zip(("dq", "dk", "dv", "ds0"), grads, ref) if g is not None])
     choose_backward(PASSES)
+    o_p, S_p = hp.raw_fwd(emu_lib, q, k, v, s, decays)
+    assert not torch.equal(S_p, S), "the forced choice made no difference: both forwards took the same kernel"
+    assert hp.error_report(o, o_p.float())["rms_ratio"] < 0.004 and hp.error_report(S, S_p.float())["rms_ratio"] < 0.006
     other = hp.raw_bwd(emu_lib, q, k, v, s, decays, d_o, None, want_ds0=want_ds0)
     for n, x, y in zip(("dq", "dk", "dv", "ds0"), grads, other):
         if x is not None:

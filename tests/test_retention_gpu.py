@@ -99,9 +99,9 @@ def test_forced_backward_choice(hip_lib, choice, B, T, H, dk, dv):
     (9, 1, 5, 128, 128, 0.5),        # single tokens
 ])
 def test_many_short_sequences_without_final_state_gradient(B, T, H, dk, dv, state_std):
-    """At most 32 tokens per sequence and nothing differentiating the final states: the backward of the suffix call
-    of the reference's POP layer (flash_pop/pop_retnet.py:163-168 discards the final states), one (sequence, head)
-    pair per step in a kernel of its own.  Oracle on the GPU, a spread of sequences."""
+    """At most 32 tokens per sequence and nothing differentiating the final states: the suffix call of the
+    reference's POP layer (flash_pop/pop_retnet.py:163-168 discards the final states), forward and backward each
+    one (sequence, head) pair per step in a kernel of its own.  Oracle on the GPU, a spread of sequences."""
     step = max(1, B // 7)
     run_plain(B, T, H, dk, dv, state_std, seed=T + B, with_ds=None, oracle_batches=list(range(0, B, step)), oracle_device=DEV)
 
