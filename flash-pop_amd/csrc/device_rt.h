@@ -79,4 +79,9 @@ FP_DEVICE u32x4 buf_load128_nt(BufView b, uint32_t off) { return __builtin_amdgc
 FP_DEVICE void buf_store128_nt(BufView b, uint32_t off, u32x4 v) { __builtin_amdgcn_raw_buffer_store_b128(v, b.rsrc, off, 0, 2); }
 FP_DEVICE void buf_store64(BufView b, uint32_t off, u32x2 v) { __builtin_amdgcn_raw_buffer_store_b64(v, b.rsrc, off, 0, 0); }
 
+// A word that another workgroup of the same launch polls (relaxed, device scope), and a short sleep between polls.
+FP_DEVICE void pace_store(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+FP_DEVICE uint32_t pace_load(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+FP_DEVICE void nap() { __builtin_amdgcn_s_sleep(8); }
+
 }  // namespace fprt

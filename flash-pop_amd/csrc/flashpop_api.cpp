@@ -49,11 +49,12 @@ bool dim_ok(int d) { return d == 64 || d == 128 || d == 192 || d == 256; }
 
 // Two measurement switches, read from the environment once per process (the first entry point that
 // looks) and changed afterwards only through fp_set_backward_choice:
-//   FLASHPOP_BWD   auto | passes | fused   which backward runs where both exist
+//   FLASHPOP_BWD   auto | passes | fused | paced   which backward runs where both exist (paced: fused, its two
+//                  workgroups per stream held together, see FusedBwdArgs::want_pace)
 //   FLASHPOP_CKPT  tokens between the checkpoints that the forward leaves for the fused backward
 //                  (a multiple of 64; 0: none; unset: 512)
 // A value that is neither is an error of every entry point, not a silent default.
-enum BwdChoice { BWD_AUTO = 0, BWD_PASSES = 1, BWD_FUSED = 2 };
+enum BwdChoice { BWD_AUTO = 0, BWD_PASSES = 1, BWD_FUSED = 2, BWD_FUSED_PACED = 3 };
 constexpr int kDefaultCheckpointEvery = 8 * fpk::CH;
 std::atomic<int> g_bwd_choice{BWD_AUTO}, g_ckpt_every{kDefaultCheckpointEvery};
 std::once_flag g_env_once;
@@ -64,8 +65,9 @@ void read_environment() {
     if (const char* e = std::getenv("FLASHPOP_BWD")) {
       if (std::strcmp(e, "passes") == 0) g_bwd_choice = BWD_PASSES;
       else if (std::strcmp(e, "fused") == 0) g_bwd_choice = BWD_FUSED;
+      else if (std::strcmp(e, "paced") == 0) g_bwd_choice = BWD_FUSED_PACED;
       else if (std::strcmp(e, "auto") != 0 && *e)
-        std::snprintf(g_env_error, sizeof g_env_error, "FLASHPOP_BWD=%.40s: expected auto, passes or fused", e);
+        std::snprintf(g_env_error, sizeof g_env_error, "FLASHPOP_BWD=%.40s: expected auto, passes, fused or paced", e);
     }
     if (const char* e = std::getenv("FLASHPOP_CKPT")) {
       char* end = nullptr;
@@ -254,7 +256,7 @@ bool use_fused_backward(const Shape& s, const void* d_blocks, bool pop_suffixes 
   read_environment();
   const int choice = g_bwd_choice.load(std::memory_order_relaxed);
   if (choice == BWD_PASSES) return false;
-  if (choice == BWD_FUSED) return true;   // whatever the length and the number of streams
+  if (choice >= BWD_FUSED) return true;   // whatever the length and the number of streams
   if (s.T < 8 * fpk::CH) return false;    // short sequences: the walk over many of them per workgroup serves better
   // Two workgroups per stream against column-tiled passes that fill the chip: the fused kernel needs enough streams.
   // Measured cross-overs on a 256-unit device (forward + backward at T = 2048 .. 4096; streams = B * H):
@@ -301,6 +303,7 @@ int backward_fused(const Shape& s, const void* q, const void* k, const void* v, 
   a.blocks_every = d_blocks ? blocks_every : 0;
   a.ckpt = in(ckpt);
   a.ckpt_every = ckpt ? ckpt_every : 0;
+  a.want_pace = g_bwd_choice.load(std::memory_order_relaxed) == BWD_FUSED_PACED;
   if (sfx) {
     a.q_sfx = in(sfx->q); a.k_sfx = in(sfx->k); a.v_sfx = in(sfx->v); a.dO_sfx = in(sg->d_o);
     a.dq_sfx = out(sg->dq); a.dk_sfx = out(sg->dk); a.dv_sfx = out(sg->dv);
@@ -849,7 +852,8 @@ int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, voi
 
 int fp_set_backward_choice(int choice, int checkpoint_every) {
   read_environment();
-  if (choice < BWD_AUTO || choice > BWD_FUSED) return fail(FP_ERR_BAD_CONFIG, "backward choice %d: expected 0 (by shape), 1 (passes) or 2 (fused)", choice);
+  if (choice < BWD_AUTO || choice > BWD_FUSED_PACED)
+    return fail(FP_ERR_BAD_CONFIG, "backward choice %d: expected 0 (by shape), 1 (passes), 2 (fused) or 3 (fused, paced)", choice);
   if (checkpoint_every >= 0 && checkpoint_every % fpk::CH != 0)
     return fail(FP_ERR_BAD_CONFIG, "the checkpoint interval must be a multiple of %d tokens (got %d)", fpk::CH, checkpoint_every);
   g_bwd_choice.store(choice, std::memory_order_relaxed);
@@ -859,6 +863,6 @@ int fp_set_backward_choice(int choice, int checkpoint_every) {
 
 const char* fp_last_error(void) { return g_err; }
 
-int fp_version(void) { return 1007; }
+int fp_version(void) { return 1008; }
 
 }  // extern "C"

@@ -161,6 +161,32 @@ int fpk_static_scratch(void** ptr, const char** err) {
   return 0;
 }
 
+// ---- pacing words of the fused backward -----------------------------------------------------------
+// One word per (batch, head) stream, through which the reverse workgroup of a stream tells the dq workgroup how
+// far it is (FusedBwdArgs::pace).  Every launch tags its values with a number of its own, so nothing is ever
+// cleared; launches that overlap on one device share the words and at worst pace each other badly.
+static __device__ __align__(256) uint32_t pace_words[fpk::PACE_SLOTS];
+
+namespace {
+std::atomic<void*> g_pace_ptr[kMaxDevices];
+std::atomic<uint32_t> g_pace_launch{1};
+
+// the words' address on the current device (nullptr: pacing stays off for this launch)
+uint32_t* pace_words_here() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = g_pace_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(pace_words)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_pace_ptr[dev].store(p, std::memory_order_release);
+  }
+  return static_cast<uint32_t*>(p);
+}
+}  // namespace
+
 int fpk_stream_is_capturing(void* stream) {
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &status) != hipSuccess) {
@@ -308,6 +334,11 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* stream, const char
   if (const char* why = fpk::check_fused_bwd(a)) {
     *err = why;
     return 1;
+  }
+  a.pace = nullptr;
+  if (fpk::fused_bwd_paces(a, fpk_compute_units())) {
+    a.pace = pace_words_here();
+    a.pace_base = g_pace_launch.fetch_add(1, std::memory_order_relaxed) << 16;
   }
   const hipStream_t st = static_cast<hipStream_t>(stream);
   if (a.dk_dim == 128 && a.dv_dim == 128) return launch_bwd_fused<128, 128>(a, 0, st, err);

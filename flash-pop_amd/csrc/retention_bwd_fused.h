@@ -505,6 +505,9 @@ FP_DEVICE void fused_bwd_reverse(const FusedBwdArgs& p, char* lds, int stream) {
     const int L = cur.L;
     const bool sfx = SFX && cur.sfx;
     const Item after = item_of(it + 2);
+    if constexpr (MODE == FB_PLAIN) {   // the loads of it + 2 chunks are on their way or done
+      if (p.pace && k.tid == 0) fprt::pace_store(p.pace + stream, p.pace_base + (uint32_t)(it + 2));
+    }
     // ---- the previous item's outputs leave (nothing writes the staging tiles before the next barrier)
     if (it > 0) {
       drain_tile<DV>(k, OUTV, p.dv, p.dv_sfx, prev);
@@ -834,12 +837,26 @@ FP_DEVICE void fused_bwd_forward(const FusedBwdArgs& p, char* lds, int stream) {
   //   2  Y^T += Z^T P^T and the outputs (output waves); the state update and the new copy of R
   //      (state waves); the next chunk's X tile
   //   3  the next chunk's W and Z tiles
+  int patience = 256;   // polls of the pacing word that this workgroup affords in all
   for (int it = 0; it < nitems; ++it) {
     const int next = SFX ? 0 : chunk_of(it + 1);
     const bool fresh = !SFX && next >= 0 && next != chunk_of(it) + 1;   // the next chunk starts another segment
     const bool sfx = SFX && cur.sfx;
     const int L = cur.L;
     const Item after = item_of(it + 2);
+    if constexpr (MODE == FB_PLAIN) {
+      // the loads that this iteration issues (behind its first barrier) open another segment: not before the reverse
+      // workgroup has asked for that segment's last chunk
+      const int c2 = chunk_of(it + 2);
+      if (p.pace && nseg > 1 && c2 >= 0 && c2 % seg_chunks == 0 && k.tid == 0) {
+        const int last = (c2 + seg_chunks < k.nch ? c2 + seg_chunks : k.nch) - 1;
+        const uint32_t want = p.pace_base + (uint32_t)(k.nch - last);
+        while (patience > 0 && (int32_t)(fprt::pace_load(p.pace + stream) - want) < 0) {
+          fprt::nap();
+          --patience;
+        }
+      }
+    }
     if (it > 0) {   // nothing writes the staging tile before the next barrier
       drain_tile<DK>(k, OUT, p.dq, p.dq_sfx, prev);
       if constexpr (FOLD) drain_suffix(it - 1);
@@ -1165,6 +1182,16 @@ FP_DEVICE void suffix_intra_bwd(const FusedBwdArgs& p, char* lds) {
 
 // The shapes the kernels above are instantiated for.
 inline bool fused_bwd_dims(int dk, int dv) { return (dk == 64 || dk == 128) && (dv == 64 || dv == 128); }
+// Pacing can only work when both workgroups of every stream are on the device at once (one workgroup per compute
+// unit), sit behind the same L2 (launch indices s and streams + s on the same XCD: streams a multiple of 8) and
+// there are checkpoints to cut the dq walk into segments.  `force`: whatever the device (the CPU harness).
+inline bool fused_bwd_paces(const FusedBwdArgs& a, int compute_units, bool force = false) {
+  if (!a.want_pace || !a.ckpt || a.ckpt_every <= 0 || a.block > 0 || a.d_blocks) return false;
+  const long long streams = (long long)a.B * a.H;
+  if (streams > PACE_SLOTS || (a.T + CH - 1) / CH >= 0xffff) return false;
+  return force || (2 * streams <= compute_units && streams % 8 == 0);
+}
+
 
 // What the kernel assumes about its arguments; nullptr or a message for the caller.
 inline const char* check_fused_bwd(const FusedBwdArgs& a) {

@@ -200,10 +200,13 @@ int fp_gated_group_norm_bwd(const void* r, const void* g, const void* d_out, voi
 /* Measurement switch; no counterpart in the reference.  Where a shape can run both the fused backward
  * kernel and the pass-per-gradient backward, the library chooses by shape; this overrides it for the
  * whole process until called again (A/B timing, tests of the path not chosen).
- *   choice            0 by shape (default), 1 always the passes, 2 the fused kernel wherever it exists
+ *   choice            0 by shape (default), 1 always the pass kernel (for the forward of sequences of at most 32
+ *                     tokens too, which otherwise has a kernel of its own), 2 the fused kernel wherever it exists,
+ *                     3 as 2 with the two workgroups of a stream paced so that they meet in the L2 (fewer bytes
+ *                     fetched, a slower launch: kept for that comparison)
  *   checkpoint_every  tokens between the states fp_retention_checkpoint_bytes asks the forward to leave:
  *                     a multiple of 64, 0 for none, negative to leave the current setting (default 512)
- * The environment variables FLASHPOP_BWD (auto | passes | fused) and FLASHPOP_CKPT give the initial
+ * The environment variables FLASHPOP_BWD (auto | passes | fused | paced) and FLASHPOP_CKPT give the initial
  * values; they are read once per process, and a value that is none of these makes every entry point
  * return FP_ERR_BAD_CONFIG.  Not synchronised with calls in flight on other threads: a forward and its
  * backward must run under the same setting. */

@@ -82,6 +82,9 @@ FP_DEVICE float sigmoid_f32(float x) { return 1.0f / (1.0f + std::exp(-x)); }
 FP_DEVICE float rsqrt_f32(float x) { return 1.0f / std::sqrt(x); }
 
 FP_DEVICE void sched_fence() {}
+FP_DEVICE void pace_store(uint32_t* p, uint32_t v) { __atomic_store_n(p, v, __ATOMIC_RELAXED); }
+FP_DEVICE uint32_t pace_load(const uint32_t* p) { return __atomic_load_n(p, __ATOMIC_RELAXED); }
+FP_DEVICE void nap() {}
 // lanes are independent OS threads here, so lane-to-lane exchange through LDS needs a real barrier
 FP_DEVICE void wave_sync() { pthread_barrier_wait(&g_lane.wave->bar); }
 FP_DEVICE float lane_xor(float v, int mask) {

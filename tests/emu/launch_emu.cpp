@@ -90,6 +90,14 @@ int fpk_launch_bwd_fused(const fpk::FusedBwdArgs& args, void* /*stream*/, const 
     *err = why;
     return 1;
   }
+  // the two workgroups of a stream run one after the other here, so the pacing words are written and read but never waited for
+  static uint32_t pace_words[fpk::PACE_SLOTS];
+  static uint32_t launches = 1;
+  a.pace = nullptr;
+  if (fpk::fused_bwd_paces(a, fpk_compute_units(), true)) {   // whatever the pretended device
+    a.pace = pace_words;
+    a.pace_base = launches++ << 16;
+  }
   if (a.dk_dim == 128 && a.dv_dim == 128) return emu_bwd_fused_128_128(a);
   if (a.dk_dim == 64 && a.dv_dim == 128) return emu_bwd_fused_64_128(a);
   if (a.dk_dim == 128 && a.dv_dim == 64) return emu_bwd_fused_128_64(a);

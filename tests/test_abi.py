@@ -31,7 +31,7 @@ def test_header_and_binding_agree(lib):
     assert names == sorted(_lib.SIGNATURES), (names, sorted(_lib.SIGNATURES))
     for n in names:
         assert hasattr(lib, n), f"{n} not exported"
-    assert lib.fp_version() == 1007
+    assert lib.fp_version() == 1008
 
 
 def test_argument_checks_return_codes(lib):
@@ -69,7 +69,7 @@ def test_argument_checks_return_codes(lib):
 
 
 def test_backward_choice_switch_checks_its_arguments(lib):
-    assert lib.fp_set_backward_choice(3, -1) == -6 and b"backward choice" in lib.fp_last_error()
+    assert lib.fp_set_backward_choice(4, -1) == -6 and b"backward choice" in lib.fp_last_error()
     assert lib.fp_set_backward_choice(0, 100) == -6 and b"multiple of 64" in lib.fp_last_error()
     assert lib.fp_set_backward_choice(1, 256) == 0
     n = ctypes.c_int(-1)
@@ -94,6 +94,7 @@ def test_environment_switches_are_validated_once():
     assert run({"FLASHPOP_BWD": "fuse"}).startswith("-6 FLASHPOP_BWD=fuse")
     assert run({"FLASHPOP_CKPT": "100"}).startswith("-6 FLASHPOP_CKPT=100")
     assert run({"FLASHPOP_BWD": "passes", "FLASHPOP_CKPT": "256"}).startswith("-1 ")
+    assert run({"FLASHPOP_BWD": "paced"}).startswith("-1 ")
 
 
 def test_python_wrappers_refuse_cpu_tensors():

@@ -30,7 +30,7 @@ def choose_backward(emu_lib):
     assert emu_lib.fp_set_backward_choice(0, 512) == 0
 
 
-PASSES, FUSED = 1, 2
+PASSES, FUSED, PACED = 1, 2, 3
 
 
 def _check_all(pairs):
@@ -207,13 +207,15 @@ def test_fused_pop_backward_that_carries_ds_once(emu_lib, choose_backward, B, nb
     (1, 330, 2, 0.5, 128, 64, 128),       # 64-wide keys
     (1, 210, 1, None, 0, 128, 64),        # 64-wide values, no checkpoints, no initial state
     (1, 300, 1, 0.3, 128, 64, 64),        # 64 x 64 states
+    (1, 330, 2, 0.5, -128, 128, 128),     # the two workgroups of a stream paced (the harness runs them in turn: no waiting)
 ])
 def test_fused_backward_with_checkpoints(emu_lib, choose_backward, B, T, H, state_std, every, dk, dv):
     """dk, dv of 64 or 128 (forced here at lengths below the eight chunks from which the library chooses it by
     itself): the backward that carries dS once, beside the
     workgroup that re-runs the state from the checkpoints the forward left (segments taken from
     the last to the first)."""
-    choose_backward(FUSED)
+    choose_backward(PACED if every < 0 else FUSED)
+    every = abs(every)
     decays = oracle.head_decays(H)
     q, k, v, s = hp.make_inputs(B, T, H, dk, dv, seed=T, state_std=state_std)
     d_o, d_s = hp.make_cotangents([(B, T, H, dv), (B, H, dk, dv)], seed=T + 1)

@@ -81,9 +81,11 @@ def test_parity_sweep(B, T, H, dk, dv, state_std):
     (2, 1, 640, 3, 64, 128),
     (1, 8, 1024, 16, 128, 128),   # the passes forced where the shape alone would take the fused backward (128 streams)
     (1, 8, 640, 12, 64, 128),
+    (3, 8, 2100, 16, 128, 128),   # the fused backward with its two workgroups per stream paced (128 streams, four checkpoints)
+    (3, 3, 1100, 8, 64, 128),     # ... 24 streams
 ])
 def test_forced_backward_choice(hip_lib, choice, B, T, H, dk, dv):
-    """fp_set_backward_choice: both backward paths of a shape against the oracle, whatever the library would pick."""
+    """fp_set_backward_choice: the backward paths of a shape against the oracle, whatever the library would pick."""
     assert hip_lib.fp_set_backward_choice(choice, -1) == 0
     try:
         run_plain(B, T, H, dk, dv, 0.1, seed=T + choice)
