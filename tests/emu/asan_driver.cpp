@@ -171,6 +171,8 @@ int main() {
   rc |= fused(1, 4, 64, 9, 1, 64, 64);        // folded suffixes of 9 tokens on 64 x 64 states
   rc |= pop(1, 256, 1, 128, 128, 64);         // gradients of block states added on the reverse walk of that kernel
   rc |= pop(1, 300, 1, 64, 128, 128);         // ... 64-wide keys, tokens after the last boundary
+  fp_set_backward_choice(3, -1);
+  rc |= checkpointed(1, 200, 2, 64, 128, 64);    // the two workgroups of a stream paced (pacing words written and polled)
   fp_set_backward_choice(0, -1);
   rc |= short_sequences(7, 16, 2, 128, 128, true);   // more pairs than workgroups, one k-step along the tokens
   rc |= short_sequences(2, 31, 1, 64, 128, true);    // two k-steps, 64-wide keys

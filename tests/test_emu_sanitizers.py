@@ -17,4 +17,4 @@ def test_all_entry_points_under_asan_and_ubsan(tmp_path):
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
     res = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=1500)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-6000:]
-    assert res.stdout.count("ok ") == 39 and "FAILED" not in res.stdout, res.stdout
+    assert res.stdout.count("ok ") == 40 and "FAILED" not in res.stdout, res.stdout
